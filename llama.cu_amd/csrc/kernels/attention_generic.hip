@@ -14,18 +14,21 @@
 // head_slopes (may be null): a bias inside the scores that grows with the distance, for position
 // encodings of that kind: slope[h] * (j - p) is added to the scaled score of key j for the query at p.
 // dv: the values' head size (the keys' is dh); out is [n, nh * dv].
+// sinks (may be null): a number per head that stands in the softmax's denominator as exp(sink[h]) beside the keys'
+// terms; it has no key, no value, no scale and no bias, and counts once for every query.
 #include "common.h"
 #include "kv_layout.h"
 
-constexpr int MAX_HEAD_DIM = 256;
+constexpr int MAX_HEAD_DIM = 640;        // NV = 4 covers values up to 256 dims, NV = 10 up to 640
 
-template <class T>
+template <class T, int NV>
 __global__ void __launch_bounds__(64)
 paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restrict__ out, int out_stride,
                                const T *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                                const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                                const int *__restrict__ req_of_token, int nh, int nkvh, int dh, int dv, int page,
-                               float scale, int window, int chunk, const float *__restrict__ head_slopes) {
+                               float scale, int window, int chunk, const float *__restrict__ head_slopes,
+                               const float *__restrict__ sinks) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int r = req_of_token[t];
     const int p = ctx_len[r] - (q_start[r + 1] - t);
@@ -42,7 +45,9 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
     const size_t page_elems = kv_page_elems(nkvh, dh, dv, page);
     const size_t v_base = kv_value_offset(nkvh, kvh, 0, 0, dh, dv, page);
     float m = -INFINITY, l = 0.f;
-    float o[MAX_HEAD_DIM / WAVE] = {0.f, 0.f, 0.f, 0.f};
+    float o[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) o[i] = 0.f;
 
     for (int base = (lo / WAVE) * WAVE; base <= p; base += WAVE) {
         const int j = base + lane;
@@ -67,7 +72,7 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
         ps[lane] = pj;
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < MAX_HEAD_DIM / WAVE; ++i) o[i] *= alpha;
+        for (int i = 0; i < NV; ++i) o[i] *= alpha;
         const int j_first = base > lo ? base : lo;
         const int j_last = base + WAVE - 1 < p ? base + WAVE - 1 : p;
         for (int j2 = j_first; j2 <= j_last; ++j2) {
@@ -75,16 +80,22 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
             const int pg = bt[j2 / page], tok = j2 % page;
             const T *vp = cache + (size_t)pg * page_elems + v_base + tok;
 #pragma unroll
-            for (int i = 0; i < MAX_HEAD_DIM / WAVE; ++i) {
+            for (int i = 0; i < NV; ++i) {
                 const int d = lane + WAVE * i;
                 if (d < dv) o[i] += pp * to_f32(vp[(size_t)d * page]);
             }
         }
         __syncthreads();
     }
-    const float inv = 1.0f / l;
+    float keep = 1.f;
+    if (sinks) {                                  // the sink's term, against the larger of the two reference points
+        const float sk = sinks[h], m_all = fmaxf(m, sk);
+        keep = expf(m - m_all);
+        l = l * keep + expf(sk - m_all);
+    }
+    const float inv = keep / l;
 #pragma unroll
-    for (int i = 0; i < MAX_HEAD_DIM / WAVE; ++i) {
+    for (int i = 0; i < NV; ++i) {
         const int d = lane + WAVE * i;
         if (d < dv) out[(size_t)t * out_stride + (size_t)h * dv + d] = from_f32<T>(o[i] * inv);
     }
@@ -99,18 +110,17 @@ LCU_API int lcu_paged_attention_generic(const void *q, int q_stride, void *out, 
                                         const void *cache, const int *block_table, int max_pages,
                                         const int *q_start, const int *ctx_len, const int *req_of_token, int n,
                                         int nh, int nkvh, int dh, int dv, int page, float scale, int window,
-                                        int chunk, const float *head_slopes, hipStream_t stream) {
+                                        int chunk, const float *head_slopes, const float *sinks, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || dh <= 0 || dh % 8 || dh > MAX_HEAD_DIM || dv <= 0 || dv > MAX_HEAD_DIM || page <= 0 || page % 8 ||
         max_pages <= 0 || window < 0 || chunk < 0 || (window > 0 && chunk > 0) || nh > 65535)
         return LCU_BAD_ARGUMENT;
     dim3 grid(n, nh), block(WAVE);
-    if (type == LCU_F32)
-        paged_attention_generic_kernel<float><<<grid, block, 0, stream>>>((const float *)q, q_stride, (float *)out, out_stride, (const float *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, chunk, head_slopes);
-    else if (type == LCU_BF16)
-        paged_attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, chunk, head_slopes);
-    else
-        return LCU_BAD_ARGUMENT;
+#define GO(T, NV) paged_attention_generic_kernel<T, NV><<<grid, block, 0, stream>>>((const T *)q, q_stride, (T *)out, out_stride, (const T *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, chunk, head_slopes, sinks)
+    if (type == LCU_F32) { if (dv <= 256) GO(float, 4); else GO(float, 10); }
+    else if (type == LCU_BF16) { if (dv <= 256) GO(bf16_t, 4); else GO(bf16_t, 10); }
+    else return LCU_BAD_ARGUMENT;
+#undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }

@@ -1,11 +1,15 @@
 // A feed-forward of many small experts of which each token uses a few.
 //
-//   route:   z = W_router h (32-bit), the `top` experts with the largest z (ties: the lower
-//            index), each with the weight sigmoid(z) (a token's weights are not made to add up to one);
+//   route:   z = W_router h (+ bias) (32-bit), the `top` experts with the largest z (ties: the lower
+//            index), each with the weight sigmoid(z) (a token's weights are not made to add up to one) or,
+//            in the other mode, with the softmax over the chosen logits alone; rows of the router's matrix
+//            behind the experts' are gates: sigmoid of their logit goes out per token;
 //   group:   the (token, choice) pairs sorted by expert and cut into tiles of up to 16 or 64 rows of
 //            one expert, on the device (nothing comes back to the host);
-//   up:      act = gelu(W_up[e] (weight * h))    the weight scales what goes INTO the expert
-//   down:    y = W_down[e] act, added to the token's output row (32-bit).
+//   up:      act = gelu(W_up[e] (weight * h))    the weight scales what goes INTO the expert; or, gated:
+//            act = silu(W_gate[e] h) * (W_up[e] h), and the weight scales what comes OUT of the expert
+//   down:    y = W_down[e] act, added to the token's output row (32-bit), in the gated form times the weight
+//            and beside a shared expert's row times its gate.
 // The products run on the matrix cores: bfloat16 operands with v_mfma_f32_16x16x32_bf16, or
 // true 32-bit with v_mfma_f32_16x16x4_f32; sums are 32-bit.  A row's result depends on that
 // row and its expert alone (never on which rows share its tile), so it does not depend on
@@ -27,11 +31,17 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 template <class T> struct alignas(8 * sizeof(T)) Row8 { T v[8]; };
 constexpr int ROUTE_CHUNKS = 8;                  // rows of up to 8 * 512 elements stay in registers
 
+// bias: null or [experts], added to the logits.  mode 0: the weight of a chosen expert is sigmoid(z); 1: the softmax over
+// the chosen logits.  extra: rows of `router` behind the experts' (at most MOE_MAX_EXTRA); gates [n, extra] takes sigmoid
+// of their logits (they are no experts and are never chosen).
+constexpr int MOE_MAX_EXTRA = 8;
 template <class T, int THREADS>
 __global__ void __launch_bounds__(THREADS)
-moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int *__restrict__ ids,
-                 float *__restrict__ wts, int d, int experts, int top) {
-    __shared__ float z[MOE_MAX_EXPERTS];
+moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, const float *__restrict__ bias, int *__restrict__ ids,
+                 float *__restrict__ wts, float *__restrict__ gates, int d, int n_experts, int top, int mode, int extra) {
+    __shared__ float z[MOE_MAX_EXPERTS + MOE_MAX_EXTRA];
+    __shared__ float zc[MOE_MAX_EXPERTS];
+    const int experts = n_experts + extra;          // rows of the router's matrix
     const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const T *row = h + (size_t)t * d;
     if (d % 8 == 0 && d <= ROUTE_CHUNKS * 512) {
@@ -60,7 +70,7 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int 
                 }
             }
             acc = wave_sum(acc);
-            if (lane == 0) z[e] = acc;
+            if (lane == 0) z[e] = acc + (bias && e < n_experts ? bias[e] : 0.f);
         }
     } else {
         for (int e = wave; e < experts; e += THREADS / WAVE) {
@@ -68,15 +78,16 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int 
             float acc = 0.f;
             for (int c = lane; c < d; c += WAVE) acc += to_f32(row[c]) * w[c];
             acc = wave_sum(acc);
-            if (lane == 0) z[e] = acc;
+            if (lane == 0) z[e] = acc + (bias && e < n_experts ? bias[e] : 0.f);
         }
     }
     __syncthreads();
+    for (int e = threadIdx.x; e < extra; e += THREADS) gates[(size_t)t * extra + e] = 1.0f / (1.0f + expf(-z[n_experts + e]));
     for (int k = 0; k < top; ++k) {                  // the first wave chooses; the others only keep the barriers
         if (wave == 0) {
             float best = -INFINITY;
             int arg = 0x7fffffff;
-            for (int e = lane; e < experts; e += WAVE) {
+            for (int e = lane; e < n_experts; e += WAVE) {
                 const float v = z[e];
                 if (v > best || (v == best && e < arg)) { best = v; arg = e; }
             }
@@ -86,14 +97,22 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int 
                 const int oa = __shfl_xor(arg, off, WAVE);
                 if (ob > best || (ob == best && oa < arg)) { best = ob; arg = oa; }
             }
-            if (arg >= experts) arg = 0;                 // every logit NaN: any expert
+            if (arg >= n_experts) arg = 0;               // every logit NaN: any expert
             if (lane == 0) {
                 ids[(size_t)t * top + k] = arg;
-                wts[(size_t)t * top + k] = 1.0f / (1.0f + expf(-z[arg]));
+                zc[k] = z[arg];
+                if (mode == 0) wts[(size_t)t * top + k] = 1.0f / (1.0f + expf(-z[arg]));
                 z[arg] = -INFINITY;
             }
         }
         __syncthreads();
+    }
+    if (mode == 1 && wave == 0) {                    // the softmax over the chosen logits (the first is the largest)
+        const float z0 = zc[0];
+        float part = 0.f;
+        for (int k = lane; k < top; k += WAVE) part += expf(zc[k] - z0);
+        const float sum = wave_sum(part);
+        for (int k = lane; k < top; k += WAVE) wts[(size_t)t * top + k] = expf(zc[k] - z0) / sum;
     }
 }
 
@@ -166,7 +185,8 @@ template <> struct Mma<float> {
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
-enum { MOE_UP = 0, MOE_DOWN = 1 };
+enum { MOE_UP = 0, MOE_DOWN = 1, MOE_UP_GATED = 2 };
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
 // Both kernels below multiply the rows of a tile (sorted rows of one expert) with that expert's matrix
 // w[e] ([N, K], row-major) on the matrix cores.  The weight is the instruction's first operand (16
@@ -177,6 +197,9 @@ enum { MOE_UP = 0, MOE_DOWN = 1 };
 //             [total, N] at the sorted row, gelu applied.
 //   MOE_DOWN: x = act [total, K] at the sorted row; out_f [total or n, N] 32-bit at the flat pair
 //             (add == 0: stored) or at the pair's token (add == 1: added; only with top == 1).
+//   MOE_UP_GATED: x = h [n, K], not scaled; w[e] holds N = 2 * features rows, in turns 16 rows of the gate matrix and the
+//             16 rows of the up matrix that meet them; out_t = act [total, N / 2] at the sorted row,
+//             silu(gate) * up.
 template <class T, int MODE>
 __device__ __forceinline__ void moe_store(const f32x4 &acc, int dst, int col0, int N, T *__restrict__ out_t,
                                           float *__restrict__ out_f, int out_stride, int add) {
@@ -207,37 +230,57 @@ moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__
     const int tile = blockIdx.x;
     if (tile >= n_tiles[0]) return;
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, g = lane / 16, l16 = lane % 16;
+    constexpr bool GATED = MODE == MOE_UP_GATED, UP = MODE != MOE_DOWN;
+    const int NF = GATED ? N / 2 : N;                // output features
     const int f0 = blockIdx.y * 64 + wave * 16;
-    if (f0 >= N) return;
+    if (f0 >= NF) return;
     const int e = tile_expert[tile], row0 = tile_begin[tile], rows = tile_rows[tile];
-    const int f = f0 + l16;
-    const T *wrow = w + (size_t)e * w_expert_stride + (size_t)(f < N ? f : N - 1) * K + g * M::PER_LANE;
+    const int f = f0 + l16 < NF ? f0 + l16 : NF - 1;
+    const int wr = GATED ? (f / 16) * 32 + f % 16 : f;       // the gate's row; the up row that meets it lies 16 further
+    const T *wrow = w + (size_t)e * w_expert_stride + (size_t)wr * K + g * M::PER_LANE;
     const bool valid = l16 < rows;
     const int srow = row0 + (valid ? l16 : 0);
     const int flat = sorted_to_flat[srow];
-    const T *xrow = (MODE == MOE_UP ? x + (size_t)(flat / top) * x_stride : x + (size_t)srow * x_stride) + g * M::PER_LANE;
+    const T *xrow = (UP ? x + (size_t)(flat / top) * x_stride : x + (size_t)srow * x_stride) + g * M::PER_LANE;
     const float sc = MODE == MOE_UP ? wts[flat] : 1.f;
-    const int dst = MODE == MOE_UP ? srow : (add ? flat / top : flat);
-    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int dst = UP ? srow : (add ? flat / top : flat);
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f}, acc2 = f32x4{0.f, 0.f, 0.f, 0.f};
     const int kfull = K / M::KSTEP * M::KSTEP;
     int k0 = 0;
     constexpr int AHEAD = 8;                         // steps of loads in flight: a wave's own arithmetic is short
     for (; k0 + AHEAD * M::KSTEP <= kfull; k0 += AHEAD * M::KSTEP) {
-        frag a[AHEAD], b[AHEAD];
+        frag a[AHEAD], b[AHEAD], a2[GATED ? AHEAD : 1];
 #pragma unroll
         for (int u = 0; u < AHEAD; ++u) a[u] = M::load(wrow + k0 + u * M::KSTEP);    // (through the caches: a load takes half of each line, the next one the other half)
+        if (GATED) {
+#pragma unroll
+            for (int u = 0; u < AHEAD; ++u) a2[GATED ? u : 0] = M::load(wrow + (size_t)16 * K + k0 + u * M::KSTEP);
+        }
 #pragma unroll
         for (int u = 0; u < AHEAD; ++u) b[u] = M::load(xrow + k0 + u * M::KSTEP);
 #pragma unroll
-        for (int u = 0; u < AHEAD; ++u) acc = M::mma(a[u], MODE == MOE_UP ? M::scaled(b[u], sc) : b[u], acc);
+        for (int u = 0; u < AHEAD; ++u) {
+            acc = M::mma(a[u], MODE == MOE_UP ? M::scaled(b[u], sc) : b[u], acc);
+            if (GATED) acc2 = M::mma(a2[GATED ? u : 0], b[u], acc2);
+        }
     }
     for (; k0 < K; k0 += M::KSTEP) {                 // the steps that are left, the last one perhaps in part
         const bool in = k0 + g * M::PER_LANE < K;
         const frag a = in ? M::load(wrow + k0) : M::zero();
         const frag b = in ? M::load(xrow + k0) : M::zero();
         acc = M::mma(a, MODE == MOE_UP ? M::scaled(b, sc) : b, acc);
+        if (GATED) acc2 = M::mma(in ? M::load(wrow + (size_t)16 * K + k0) : M::zero(), b, acc2);
     }
-    if (valid) moe_store<T, MODE>(acc, dst, f0 + 4 * g, N, out_t, out_f, out_stride, add);
+    if (!valid) return;
+    if (GATED) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int col = f0 + 4 * g + i;
+            if (col < NF) out_t[(size_t)dst * out_stride + col] = from_f32<T>(silu_f(acc[i]) * acc2[i]);
+        }
+    } else {
+        moe_store<T, MODE>(acc, dst, f0 + 4 * g, N, out_t, out_f, out_stride, add);
+    }
 }
 
 // Many rows an expert (prompts): tiles of up to 64 rows; a block of four waves takes a tile and 128
@@ -274,10 +317,10 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
     for (int i = 0; i < 2; ++i) {
         const int r = tid / CH + 32 * i;
         const int srow = row0 + (r < rows ? r : 0);
-        if (MODE == MOE_UP) {
+        if (MODE != MOE_DOWN) {
             const int flat = sorted_to_flat[srow];
             xptr[i] = x + (size_t)(flat / top) * x_stride + ch * PL;
-            xsc[i] = wts[flat];
+            xsc[i] = MODE == MOE_UP ? wts[flat] : 1.f;
         } else {
             xptr[i] = x + (size_t)srow * x_stride + ch * PL;
             xsc[i] = 1.f;
@@ -342,19 +385,30 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
             const int flat = sorted_to_flat[srow];
             dst = add ? flat / top : flat;
         }
+        if (MODE == MOE_UP_GATED) {                 // the wave's first 16 rows are a gate block, its second the up block that meets it
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = (n0 + 32 * wave) / 2 + 4 * g + i;
+                if (col < N / 2) out_t[(size_t)dst * out_stride + col] = from_f32<T>(silu_f(acc[0][m][i]) * acc[1][m][i]);
+            }
+            continue;
+        }
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
-            moe_store<T, MODE>(acc[ft][m], dst, n0 + 32 * wave + 16 * ft + 4 * g, N, out_t, out_f, out_stride, add);
+            moe_store<T, MODE == MOE_UP_GATED ? MOE_UP : MODE>(acc[ft][m], dst, n0 + 32 * wave + 16 * ft + 4 * g, N, out_t, out_f, out_stride, add);
     }
 }
 
-// out[t, c] += sum_k y[t * top + k, c]  (in the order of k)
-__global__ void moe_combine_kernel(float *__restrict__ out, const float *__restrict__ y, int n, int d, int top) {
+// out[t, c] += sum_k wts[t, k] * y[t * top + k, c]  (in the order of k; wts null: ones)  + gate[t] * shared[t, c]  (shared null: nothing)
+template <class T>
+__global__ void moe_combine_kernel(float *__restrict__ out, const float *__restrict__ y, const float *__restrict__ wts,
+                                   const T *__restrict__ shared, const float *__restrict__ gate, int n, int d, int top) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= d) return;
     for (size_t t = blockIdx.y; t < (size_t)n; t += gridDim.y) {
         float acc = out[t * d + c];
-        for (int k = 0; k < top; ++k) acc += y[(t * top + k) * d + c];
+        for (int k = 0; k < top; ++k) acc += (wts ? wts[t * top + k] : 1.f) * y[(t * top + k) * d + c];
+        if (shared) acc += (gate ? gate[t] : 1.f) * to_f32(shared[t * d + c]);
         out[t * d + c] = acc;
     }
 }
@@ -364,12 +418,16 @@ __global__ void moe_combine_kernel(float *__restrict__ out, const float *__restr
 LCU_API int lcu_moe_tile_rows(int total, int experts) { return (long long)total <= 16ll * experts ? 16 : MOE_TILE_ROWS; }
 
 // h: [n, d] of `type`; router: [experts, d] 32-bit; ids, wts: [n * top].
-LCU_API int lcu_moe_route(const void *h, int type, const float *router, int *ids, float *wts, int n, int d, int experts,
-                          int top, hipStream_t stream) {
+// bias: null or [experts] 32-bit; mode 0: sigmoid weights, 1: softmax over the chosen; extra, gates: see the kernel
+// (router then has experts + extra rows).
+LCU_API int lcu_moe_route(const void *h, int type, const float *router, const float *bias, int *ids, float *wts, float *gates,
+                          int n, int d, int experts, int top, int mode, int extra, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
-    if (d <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts) return LCU_BAD_ARGUMENT;
+    if (d <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts || (mode != 0 && mode != 1) ||
+        extra < 0 || extra > MOE_MAX_EXTRA || (extra && !gates))
+        return LCU_BAD_ARGUMENT;
     const bool few = n <= 256 && experts > 4;
-#define GO(T, TH) moe_route_kernel<T, TH><<<dim3(n), dim3(TH), 0, stream>>>((const T *)h, router, ids, wts, d, experts, top)
+#define GO(T, TH) moe_route_kernel<T, TH><<<dim3(n), dim3(TH), 0, stream>>>((const T *)h, router, bias, ids, wts, gates, d, experts, top, mode, extra)
     if (type == LCU_F32) { if (few) GO(float, 1024); else GO(float, 256); }
     else if (type == LCU_BF16) { if (few) GO(bf16_t, 1024); else GO(bf16_t, 256); }
     else return LCU_BAD_ARGUMENT;
@@ -381,30 +439,39 @@ LCU_API int lcu_moe_route(const void *h, int type, const float *router, int *ids
 // ints: scratch of total + 3 * max_tiles + 1 entries, laid out as sorted_to_flat, tile_expert, tile_begin,
 // tile_rows, n_tiles.
 // w_up: [experts, ff, d], w_down: [experts, d, ff] of `type`.  act: scratch [total, ff] of `type`; y: scratch
-// [total, d] 32-bit (only read and written when top > 1).  out: [n, d] 32-bit, added to.
+// [total, d] 32-bit (only read and written when top > 1 or gated).  out: [n, d] 32-bit, added to.
+// gated: w_up is [experts, 2 * ff, d], in turns 16 rows of the gate matrix and the 16 rows of the up matrix that meet
+// them (ff a multiple of 16); act = silu(gate h) * (up h), and the weight scales what comes out.  shared (null or
+// [n, d] of `type`) with shared_gate (null or [n] 32-bit): rows that are added beside the experts', times the gate.
 LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float *wts, int *ints, int max_tiles,
                             const void *w_up, const void *w_down, void *act, float *y, float *out, int n, int d, int ff,
-                            int experts, int top, hipStream_t stream) {
+                            int experts, int top, int gated, const void *shared, const float *shared_gate, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     const int per = type == LCU_BF16 ? 8 : 4;
     if (d <= 0 || ff <= 0 || d % per || ff % per || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || max_tiles <= 0 ||
-        (type != LCU_F32 && type != LCU_BF16))
+        (type != LCU_F32 && type != LCU_BF16) || (gated && ff % 16) || (shared && !gated))
         return LCU_BAD_ARGUMENT;
     const int total = n * top;
     const int tile_rows = lcu_moe_tile_rows(total, experts);
     int *sorted = ints, *t_exp = ints + total, *t_beg = t_exp + max_tiles, *t_rows = t_beg + max_tiles, *n_tiles = t_rows + max_tiles;
     moe_group_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, total, experts, sorted, t_exp, t_beg, t_rows, n_tiles, max_tiles, tile_rows);
     LCU_LAUNCH_CHECK();
-    const int add = top == 1;
+    const int add = top == 1 && !gated;
     float *down_to = add ? out : y;
+    if (!add && !y) return LCU_BAD_ARGUMENT;
     const int per_block = tile_rows == 16 ? 64 : 128;         // features a block takes
     dim3 block(256), gu(max_tiles, (ff + per_block - 1) / per_block), gd(max_tiles, (d + per_block - 1) / per_block);
+    const int up_rows = gated ? 2 * ff : ff;                  // rows of an expert's first matrix
     if (tile_rows != 16) {                                    // a flat grid: the kernel shares it out over the dies itself
-        gu = dim3(8 * max_tiles * (((ff + 127) / 128 + 7) / 8));
+        gu = dim3(8 * max_tiles * (((up_rows + 127) / 128 + 7) / 8));
         gd = dim3(8 * max_tiles * (((d + 127) / 128 + 7) / 8));
     }
 #define GO(KERNEL, T)                                                                                                              \
-    KERNEL<T, MOE_UP><<<gu, block, 0, stream>>>((const T *)h, d, (const T *)w_up, (size_t)ff * d, ff, d, sorted, wts, t_exp, t_beg, \
+    if (gated)                                                                                                                     \
+        KERNEL<T, MOE_UP_GATED><<<gu, block, 0, stream>>>((const T *)h, d, (const T *)w_up, (size_t)up_rows * d, up_rows, d, sorted, wts, \
+                                                      t_exp, t_beg, t_rows, n_tiles, max_tiles, (T *)act, nullptr, ff, top, 0);       \
+    else                                                                                                                           \
+        KERNEL<T, MOE_UP><<<gu, block, 0, stream>>>((const T *)h, d, (const T *)w_up, (size_t)ff * d, ff, d, sorted, wts, t_exp, t_beg, \
                                                 t_rows, n_tiles, max_tiles, (T *)act, nullptr, ff, top, 0);                         \
     KERNEL<T, MOE_DOWN><<<gd, block, 0, stream>>>((const T *)act, ff, (const T *)w_down, (size_t)ff * d, d, ff, sorted, wts, t_exp, \
                                                   t_beg, t_rows, n_tiles, max_tiles, nullptr, down_to, d, top, add)
@@ -416,7 +483,9 @@ LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float
 #undef GO
     LCU_LAUNCH_CHECK();
     if (!add) {
-        moe_combine_kernel<<<dim3((d + 255) / 256, n < 65535 ? n : 65535), dim3(256), 0, stream>>>(out, y, n, d, top);
+        const dim3 gc((d + 255) / 256, n < 65535 ? n : 65535);
+        if (type == LCU_BF16) moe_combine_kernel<bf16_t><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const bf16_t *)shared, shared_gate, n, d, top);
+        else moe_combine_kernel<float><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const float *)shared, shared_gate, n, d, top);
         LCU_LAUNCH_CHECK();
     }
     return LCU_OK;

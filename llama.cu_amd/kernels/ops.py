@@ -309,30 +309,35 @@ def _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, 
     return n
 
 
+GENERIC_MAX_HEAD_DIM = 640      # what the generic attention kernel takes for keys and for values
+
+
 def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
                             q_start: torch.Tensor, ctx_len: torch.Tensor, req_of_token: torch.Tensor,
                             n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, scale: float,
                             window: int = 0, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0,
-                            chunk: int = 0) -> torch.Tensor:
+                            chunk: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of the step's queries over the paged cache (every shape).  ``head_slopes``
     (float32 [n_heads]) adds ``slope[h] * (key position - query position)`` to the scaled scores.
     ``value_dim``: the values' head size if it is not the keys' (``out`` is ``[n, n_heads * value_dim]``).
-    ``chunk``: the query at position ``p`` sees the keys from ``p - p % chunk`` on only (instead of a window)."""
+    ``chunk``: the query at position ``p`` sees the keys from ``p - p % chunk`` on only (instead of a window).
+    ``sinks`` (float32 [n_heads]): ``exp(sink[h])`` stands in every softmax's denominator beside the keys' terms."""
     n = _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size, value_dim)
     value_dim = value_dim or head_dim
-    if head_dim % 8 or head_dim > 256 or value_dim > 256:
-        raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 8, and it and the values' {value_dim} at most 256")
-    if head_slopes is not None:
-        _gpu(head_slopes)
-        if head_slopes.dtype != torch.float32 or head_slopes.shape != (n_heads,) or not head_slopes.is_contiguous():
-            raise KernelError(f"attention: head_slopes must be contiguous float32 [{n_heads}], got {head_slopes.dtype} {tuple(head_slopes.shape)}")
+    if head_dim % 8 or head_dim > GENERIC_MAX_HEAD_DIM or value_dim > GENERIC_MAX_HEAD_DIM:
+        raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 8, and it and the values' {value_dim} at most {GENERIC_MAX_HEAD_DIM}")
+    for vec, what in ((head_slopes, "head_slopes"), (sinks, "sinks")):
+        if vec is not None:
+            _gpu(vec)
+            if vec.dtype != torch.float32 or vec.shape != (n_heads,) or not vec.is_contiguous():
+                raise KernelError(f"attention: {what} must be contiguous float32 [{n_heads}], got {vec.dtype} {tuple(vec.shape)}")
     lib = build.load("attention_generic")
     _check(lib.lcu_paged_attention_generic(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _type(q, "q"), _ptr(cache),
                                            _ptr(block_table), block_table.shape[1], _ptr(q_start), _ptr(ctx_len),
                                            _ptr(req_of_token), n, n_heads, n_kv_heads, head_dim, value_dim, page_size,
-                                           ctypes.c_float(scale), int(window), int(chunk), _ptr(head_slopes), _stream()),
-           "paged_attention_generic")
+                                           ctypes.c_float(scale), int(window), int(chunk), _ptr(head_slopes), _ptr(sinks),
+                                           _stream()), "paged_attention_generic")
     return out
 
 
@@ -558,7 +563,7 @@ def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
                     n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0,
                     force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0,
-                    chunk: int = 0) -> torch.Tensor:
+                    chunk: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
     ``group``: picks the kernel for the batch's shape and type.  ``chunk``: keys of the query's own chunk of so many
     positions only (the matrix-core kernels take it as a negative window).  With a bias inside the scores
@@ -570,10 +575,10 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
             raise KernelError(f"attention: head_slopes must be contiguous float32 [{n_heads}]")
     if chunk and window:
         raise KernelError("attention: a window and chunks together are not supported")
-    if force_generic or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
+    if force_generic or sinks is not None or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
             or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
         return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
-                                       n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim, chunk)
+                                       n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim, chunk, sinks)
     n = _attention_args(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size)
     if chunk:
@@ -1157,81 +1162,121 @@ def delta_rule(proj: torch.Tensor, offsets: Dict[str, int], w2_t: torch.Tensor, 
 # ------------------------------------------------------------------ mixture of experts
 
 
-def moe_route(h: torch.Tensor, router: torch.Tensor, top: int):
-    """``(ids, weights)``, each ``[n, top]``: every row's ``top`` experts by ``router @ h`` (32-bit; ties go to the
-    lower index), largest first, with the weight ``sigmoid`` of that logit."""
-    _gpu(h, router)
+def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, bias: Optional[torch.Tensor] = None, softmax_chosen: bool = False,
+              extra: int = 0):
+    """``(ids, weights)``, each ``[n, top]``: every row's ``top`` experts by ``router @ h + bias`` (32-bit; ties go to the
+    lower index), largest first, with the weight ``sigmoid`` of that logit or, with ``softmax_chosen``, the softmax over
+    the chosen logits alone.  ``extra``: the last ``extra`` rows of ``router`` are no experts but gates; then a third
+    result ``[n, extra]`` holds ``sigmoid`` of their logits."""
+    _gpu(h, router, bias)
     _rows(h, "moe input"); _contig(h, "moe input"); _contig(router, "router")
     n, d = h.shape
     if router.dtype != torch.float32 or router.dim() != 2 or router.shape[1] != d:
         raise KernelError(f"moe_route: the router must be float32 [experts, {d}], got {router.dtype} {tuple(router.shape)}")
-    experts = router.shape[0]
-    if not 0 < top <= experts or experts > 1024:
-        raise KernelError(f"moe_route: top {top} of {experts} experts is not supported (at most 1024 experts)")
+    experts = router.shape[0] - int(extra)
+    if not 0 < top <= experts or experts > 1024 or not 0 <= extra <= 8:
+        raise KernelError(f"moe_route: top {top} of {experts} experts is not supported (at most 1024 experts, 8 gates)")
+    _f32_vec(bias, "router bias", experts)
     ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
     wts = torch.empty((n, top), dtype=torch.float32, device=h.device)
+    gates = torch.empty((n, extra), dtype=torch.float32, device=h.device) if extra else None
     lib = build.load("moe")
-    _check(lib.lcu_moe_route(_ptr(h), _type(h, "moe input"), _ptr(router), _ptr(ids), _ptr(wts), n, d, experts, top, _stream()),
-           "moe_route")
-    return ids, wts
+    _check(lib.lcu_moe_route(_ptr(h), _type(h, "moe input"), _ptr(router), _ptr(bias), _ptr(ids), _ptr(wts), _ptr(gates), n, d,
+                             experts, top, int(bool(softmax_chosen)), int(extra), _stream()), "moe_route")
+    return (ids, wts, gates) if extra else (ids, wts)
 
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
-                out: torch.Tensor) -> torch.Tensor:
+                out: torch.Tensor, gated: bool = False, shared: Optional[torch.Tensor] = None,
+                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[t] += sum over t's experts e of  w_down[e] @ gelu(w_up[e] @ (weight * h[t]))`` (the exact gelu; the
     weight scales what goes INTO the expert, not what comes out).  ``w_up [experts, ff, d]``, ``w_down [experts, d, ff]`` in ``h``'s type,
-    ``out`` float32 ``[n, d]``."""
-    _gpu(h, ids, wts, w_up, w_down, out)
+    ``out`` float32 ``[n, d]``.  ``gated``: ``out[t] += sum_e weight * w_down[e] @ (silu(gate[e] @ h[t]) * (up[e] @ h[t]))``
+    with ``w_up [experts, 2 * ff, d]`` holding in turns 16 rows of the gate matrix and the 16 up rows that meet them
+    (``gated_rows`` lays them out so); ``shared [n, d]`` (with ``shared_gate [n]`` float32, or ones) is added beside."""
+    _gpu(h, ids, wts, w_up, w_down, out, shared, shared_gate)
     _rows(h, "moe input")
     for t, what in ((h, "moe input"), (ids, "moe ids"), (wts, "moe weights"), (w_up, "moe up"), (w_down, "moe down"), (out, "moe out")):
         _contig(t, what)
     n, d = h.shape
-    if w_up.dim() != 3 or w_down.dim() != 3 or w_up.shape[2] != d or w_down.shape != (w_up.shape[0], d, w_up.shape[1]) \
+    experts, ff = w_down.shape[0], w_down.shape[2] if w_down.dim() == 3 else 0
+    if w_up.dim() != 3 or w_down.dim() != 3 or w_up.shape != (experts, (2 if gated else 1) * ff, d) or w_down.shape[1] != d \
             or w_up.dtype != h.dtype or w_down.dtype != h.dtype:
         raise KernelError(f"moe_experts: up {tuple(w_up.shape)} {w_up.dtype} and down {tuple(w_down.shape)} {w_down.dtype} do not fit rows of {d} {h.dtype}")
-    experts, ff = w_up.shape[0], w_up.shape[1]
     top = ids.shape[1] if ids.dim() == 2 else 0
     if ids.shape != (n, top) or ids.dtype != torch.int32 or wts.shape != (n, top) or wts.dtype != torch.float32 or top < 1:
         raise KernelError("moe_experts: ids (int32) and weights (float32) must be [n, top]")
     if out.shape != (n, d) or out.dtype != torch.float32:
         raise KernelError("moe_experts: out must be float32 [n, d]")
     per = 8 if h.dtype == torch.bfloat16 else 4
-    if d % per or ff % per:
-        raise KernelError(f"moe_experts: the width {d} and the experts' {ff} must be multiples of {per}")
+    if d % per or ff % (16 if gated else per):
+        raise KernelError(f"moe_experts: the width {d} and the experts' {ff} must be multiples of {per} ({16 if gated else per} for the experts')")
+    if shared is not None:
+        _contig(shared, "shared expert rows")
+        if not gated or shared.shape != (n, d) or shared.dtype != h.dtype:
+            raise KernelError("moe_experts: shared rows go with gated experts and must be [n, d] of the input's type")
+        if shared_gate is not None and (shared_gate.dtype != torch.float32 or shared_gate.numel() != n or not shared_gate.is_contiguous()):
+            raise KernelError("moe_experts: the shared rows' gate must be contiguous float32 [n]")
     lib = build.load("moe")
     total = n * top
     tile = lib.lcu_moe_tile_rows(total, experts)
     max_tiles = min(total, total // tile + experts)
     ints = torch.empty(total + 3 * max_tiles + 1, dtype=torch.int32, device=h.device)
     act = torch.empty((total, ff), dtype=h.dtype, device=h.device)
-    y = torch.empty((total, d), dtype=torch.float32, device=h.device) if top > 1 else None
+    y = torch.empty((total, d), dtype=torch.float32, device=h.device) if (top > 1 or gated) else None
     _check(lib.lcu_moe_experts(_ptr(h), _type(h, "moe input"), _ptr(ids), _ptr(wts), _ptr(ints), max_tiles, _ptr(w_up),
-                               _ptr(w_down), _ptr(act), _ptr(y), _ptr(out), n, d, ff, experts, top, _stream()), "moe_experts")
+                               _ptr(w_down), _ptr(act), _ptr(y), _ptr(out), n, d, ff, experts, top, int(bool(gated)),
+                               _ptr(shared), _ptr(shared_gate if shared is not None else None), _stream()), "moe_experts")
     return out
+
+
+def gated_rows(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``gate, up [experts, ff, d]`` (ff a multiple of 16) as the gated experts' first matrix ``[experts, 2 * ff, d]``: in
+    turns 16 rows of the gate matrix and the 16 rows of the up matrix that meet them."""
+    e, ff, d = gate.shape
+    if up.shape != gate.shape or ff % 16:
+        raise KernelError(f"gated_rows: gate {tuple(gate.shape)} and up {tuple(up.shape)} must agree, with a multiple of 16 rows")
+    return torch.stack([gate.view(e, ff // 16, 16, d), up.view(e, ff // 16, 16, d)], dim=2).reshape(e, 2 * ff, d).contiguous()
 
 
 # ------------------------------------------------------------------ norms behind a sublayer
 
 
 def norm_post(x: torch.Tensor, a: torch.Tensor, w_post: torch.Tensor, eps_post: float, w_pre: Optional[torch.Tensor] = None,
-              eps_pre: float = 0.0, out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+              eps_pre: float = 0.0, out_dtype: Optional[torch.dtype] = None, a_bias: Optional[torch.Tensor] = None,
+              copy: Optional[bool] = None) -> Optional[torch.Tensor]:
     """``x += a * rsqrt(mean(a^2) + eps_post) * w_post`` (``x``: the float32 residual stream, in place; ``a``: a
     sublayer's output) and, with ``w_pre``, the rows ``x * rsqrt(mean(x^2) + eps_pre) * w_pre`` of the norm that
-    follows, in ``out_dtype``; one kernel.  The weights are float32 factors."""
-    _gpu(x, a, w_post, w_pre)
+    follows, in ``out_dtype``; one kernel.  The weights are float32 factors.  ``copy`` (without ``w_pre``; taken as
+    asked for where ``out_dtype`` is given without ``w_pre``): the new stream itself comes back, rounded to
+    ``out_dtype``, for a sublayer that reads the stream without a norm.
+    ``a_bias`` (float32 ``[d]``): a bias that ``a`` still lacks; ``a + a_bias`` is what is normed."""
+    _gpu(x, a, w_post, w_pre, a_bias)
     _rows(x, "residual stream"); _contig(x, "residual stream"); _contig(a, "sublayer output")
     n, d = x.shape
     if x.dtype != torch.float32 or a.shape != (n, d):
         raise KernelError(f"norm_post: the stream must be float32 and the sublayer's output of its shape, got {x.dtype} {tuple(x.shape)} and {tuple(a.shape)}")
-    _f32_vec(w_post, "norm weight", d); _f32_vec(w_pre, "norm weight", d)
+    _f32_vec(w_post, "norm weight", d); _f32_vec(w_pre, "norm weight", d); _f32_vec(a_bias, "output bias", d)
     out = None
-    if w_pre is not None:
+    if copy is None:
+        copy = w_pre is None and out_dtype is not None
+    if w_pre is not None or copy:
         out = torch.empty((n, d), dtype=out_dtype or a.dtype, device=x.device)
     lib = build.load("norm_post")
-    _check(lib.lcu_norm_post(_ptr(x), _ptr(a), _type(a, "sublayer output"), _ptr(w_post), ctypes.c_float(eps_post), _ptr(w_pre),
-                             ctypes.c_float(eps_pre), _ptr(out), _type(out, "norm out") if out is not None else F32, n, d,
-                             _stream()), "norm_post")
+    _check(lib.lcu_norm_post(_ptr(x), _ptr(a), _type(a, "sublayer output"), _ptr(a_bias), _ptr(w_post), ctypes.c_float(eps_post),
+                             _ptr(w_pre), ctypes.c_float(eps_pre), _ptr(out), _type(out, "norm out") if out is not None else F32,
+                             n, d, _stream()), "norm_post")
     return out
+
+
+def row_bias(rows: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """``rows[t] += bias`` in place (``bias``: float32 over the columns; the sum is 32-bit, rounded once)."""
+    _gpu(rows, bias)
+    _rows(rows, "rows"); _contig(rows, "rows")
+    _f32_vec(bias, "bias", rows.shape[1])
+    lib = build.load("norm_post")
+    _check(lib.lcu_row_bias(_ptr(rows), _type(rows, "rows"), _ptr(bias), rows.shape[0], rows.shape[1], _stream()), "row_bias")
+    return rows
 
 
 def scaled_sum(acc: Optional[torch.Tensor], x: torch.Tensor, scale: float) -> torch.Tensor:
@@ -1309,6 +1354,47 @@ def head_gate(out: torch.Tensor, gate_rows: torch.Tensor, g_off: int, n_heads: i
     _check(lib.lcu_head_gate(_ptr(out), _type(out, "attention out"), _ptr(gate_rows), _type(gate_rows, "gate rows"),
                              gate_rows.stride(0), int(g_off), n, n_heads, value_dim, _stream()), "head_gate")
     return out
+
+
+def latent_prepare(rows: torch.Tensor, q_out: torch.Tensor, n_heads: int, q_head_stride: int, q_rot_off: int, kv_off: int,
+                   rank: int, rot: int, stored_dim: int, stored_value_dim: int, positions: torch.Tensor, cos: torch.Tensor,
+                   sin: torch.Tensor, c_norm: Optional[torch.Tensor] = None, eps: float = 0.0,
+                   cache: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None, page_size: int = 16) -> torch.Tensor:
+    """Latent attention between its input product and the attention over the cache.  ``rows [n, *]``: query head ``h``'s
+    turned part at column ``h * q_head_stride + q_rot_off`` (``rot`` columns), the latent product at ``kv_off`` (``rank +
+    rot`` columns).  ``q_out [n, n_heads * stored_dim]`` holds every head's folded plain part in its first ``rank``
+    columns already; the rotated turned part is written behind it, zeros behind that.  With ``cache``: the latent's first
+    ``rank`` columns, divided by their root mean square and multiplied by ``c_norm`` (float32), and the rotated last ``rot``
+    go to the token's place in its page as the one key head ``[c, r]`` (``stored_dim`` dims) with the value ``c``
+    (``stored_value_dim`` dims).  The rotation pairs dim ``i`` with ``i + rot / 2``."""
+    _gpu(rows, q_out, positions, cos, sin, c_norm, cache, slots)
+    _rows(rows, "latent rows"); _rows(q_out, "folded queries"); _contig(q_out, "folded queries")
+    n, width = rows.shape
+    store = cache is not None
+    if q_out.shape != (n, n_heads * stored_dim) or stored_dim % 8 or rank + rot > stored_dim or stored_value_dim < rank \
+            or max(stored_dim, stored_value_dim) > 640 or rot % 2 or rot < 2:
+        raise KernelError(f"latent_prepare: queries {tuple(q_out.shape)} do not fit {n_heads} heads of {stored_dim} holding {rank} + {rot}")
+    if q_rot_off < 0 or (n_heads - 1) * q_head_stride + q_rot_off + rot > width or (store and (kv_off < 0 or kv_off + rank + rot > width)):
+        raise KernelError(f"latent_prepare: the turned parts or the latent lie outside the rows' {width} columns")
+    if cos.shape != sin.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.dim() != 2 or cos.shape[1] * 2 != rot \
+            or not cos.is_contiguous() or not sin.is_contiguous():
+        raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, rot/2]")
+    _i32(positions, "positions", n)
+    if store:
+        _f32_vec(c_norm, "latent norm weight", rank)
+        if c_norm is None:
+            raise KernelError("latent_prepare: the cache write needs the latent's norm weight")
+        _i32(slots, "cache slots", n)
+        _contig(cache, "cache")
+        if cache.dtype != q_out.dtype or cache.dim() != 3 or cache.shape[1] * cache.shape[2] != (stored_dim + stored_value_dim) * page_size:
+            raise KernelError(f"cache: {cache.dtype} {tuple(cache.shape)} does not hold pages of ({stored_dim} + {stored_value_dim}) x {page_size} {q_out.dtype}")
+    lib = build.load("latent")
+    _check(lib.lcu_latent_prepare(_ptr(rows), _type(rows, "latent rows"), n, rows.stride(0), int(q_head_stride), int(q_rot_off),
+                                  int(kv_off), _ptr(c_norm), ctypes.c_float(eps), _ptr(positions), _ptr(cos), _ptr(sin),
+                                  cos.shape[0], _ptr(q_out), _type(q_out, "folded queries"), _ptr(slots), _ptr(cache), n_heads,
+                                  int(rank), int(rot), int(stored_dim), int(stored_value_dim), int(page_size), int(store),
+                                  _stream()), "latent_prepare")
+    return q_out
 
 
 # ------------------------------------------------------------------ retention

@@ -25,14 +25,22 @@ class Attention(Part):
     # the tensors' names under the part's own, as files with config.json's names hold them; ``names`` replaces any
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias",
-             "v_bias": "v_proj.bias", "q_head_norm": "q_head_norm.weight", "k_head_norm": "k_head_norm.weight", "g": "g_proj.weight"}
+             "v_bias": "v_proj.bias", "q_head_norm": "q_head_norm.weight", "k_head_norm": "k_head_norm.weight", "g": "g_proj.weight",
+             "sink": "sinks", "o_bias": "o_proj.bias"}
 
     def __init__(self, hidden_size: int, heads: int, kv_heads: int, head_dim: int, scale: Optional[float] = None,
                  window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False, page_size: int = 0,
                  value_dim: int = 0, projection_norm_eps: Optional[float] = None, query_temperature=None,
                  names: Optional[Dict[str, str]] = None, bias: bool = False, head_norm_eps: Optional[float] = None,
-                 chunk: int = 0, head_gate: bool = False):
-        """``bias``: q, k and v have biases (tensors ``q_bias``, ``k_bias``, ``v_bias``), added in the projection.
+                 chunk: int = 0, head_gate: bool = False, values_are_keys: bool = False, head_norm_weight: bool = True,
+                 sink: bool = False, out_bias: bool = False):
+        """``values_are_keys``: there is no value projection; a token's values are its keys as projected (with their bias,
+        before any norm or rotation).  ``head_norm_weight=False``: the norm per head has no weight.  ``sink``: a learned
+        number per head (tensor ``sink`` ``[heads]``) stands in the softmax's denominator as ``exp(sink)``, with no key,
+        value, scale or bias.  ``out_bias``: the output projection has a bias (tensor ``o_bias``); ``forward(...,
+        bias_later=True)`` leaves it to the caller (``output_bias``), who adds it where it reads the rows anyway.  With a
+        position encoding that is a bias inside the scores the general path hands its slopes to the attention kernel.
+        ``bias``: q, k and v have biases (tensors ``q_bias``, ``k_bias``, ``v_bias``), added in the projection.
         ``head_norm_eps``: every q and k head is divided by its root mean square and multiplied by a weight over the
         head's dims that all heads share (tensors ``q_head_norm``, ``k_head_norm``), before any rotation.  ``chunk``: the
         query at position ``p`` sees only the keys from ``p - p % chunk`` on (instead of a window).  ``head_gate``: each
@@ -63,6 +71,11 @@ class Attention(Part):
             self.q_temp = (float(coef), int(every))
         self.names = dict(self.NAMES, **(names or {}))
         self.bias, self.head_gate = bool(bias), bool(head_gate)
+        self.values_are_keys, self.head_norm_weight = bool(values_are_keys), bool(head_norm_weight)
+        self.sink, self.out_bias = bool(sink), bool(out_bias)
+        if self.values_are_keys and self.value_dim != self.head_dim:
+            raise ValueError("attention: values that are the keys have the keys' head size")
+        self.sinks = self.output_bias = None
         self.head_norm_eps = None if head_norm_eps is None else float(head_norm_eps)
         self.chunk = int(chunk or 0)
         if self.chunk and self.window:
@@ -78,6 +91,7 @@ class Attention(Part):
         self.graph_safe = self.position.graph_safe
         rot = self.position.rotated_dims()
         self.general = bool(self.bias or self.head_gate or self.head_norm_eps is not None or self.chunk
+                            or self.values_are_keys or self.sink or self.out_bias
                             or (rot and (self.value_dim != self.head_dim or self.padded_dim != self.head_dim)))
         if self.general and (self.shares_kv or self.norm_eps is not None or self.q_temp is not None):
             raise ValueError("attention: biases, head norms, chunks, a head gate or values of their own size under a rotation "
@@ -92,7 +106,8 @@ class Attention(Part):
         t = {nm["q"]: TensorSpec((nh * dh, d)), nm["o"]: TensorSpec((d, nh * dv))}
         if not self.shares_kv:
             t[nm["k"]] = TensorSpec((nkv * dh, d))
-            t[nm["v"]] = TensorSpec((nkv * dv, d))
+            if not self.values_are_keys:
+                t[nm["v"]] = TensorSpec((nkv * dv, d))
         if self.norm_eps is not None:
             t[nm["q_norm"]] = TensorSpec((nh * dh,), init="one_plus_normal")
             if not self.shares_kv:
@@ -100,8 +115,13 @@ class Attention(Part):
         if self.bias:
             t[nm["q_bias"]] = TensorSpec((nh * dh,))
             t[nm["k_bias"]] = TensorSpec((nkv * dh,))
-            t[nm["v_bias"]] = TensorSpec((nkv * dv,))
-        if self.head_norm_eps is not None:
+            if not self.values_are_keys:
+                t[nm["v_bias"]] = TensorSpec((nkv * dv,))
+        if self.sink:
+            t[nm["sink"]] = TensorSpec((nh,))
+        if self.out_bias:
+            t[nm["o_bias"]] = TensorSpec((d,))
+        if self.head_norm_eps is not None and self.head_norm_weight:
             t[nm["q_head_norm"]] = TensorSpec((dh,), init="one_plus_normal")
             t[nm["k_head_norm"]] = TensorSpec((dh,), init="one_plus_normal")
         if self.head_gate:
@@ -110,10 +130,14 @@ class Attention(Part):
 
     def fused_groups(self, dtype, device):
         if self.general:
-            return [(tuple(self.names[k] for k in ("q", "k", "v") + (("g",) if self.head_gate else ())), 0)]
+            return [(tuple(self.names[k] for k in self._in_keys()), 0)]
         if self.shares_kv or self.padded_dim != self.head_dim:
             return []
         return [((self.names["q"], self.names["k"], self.names["v"]), 0)]
+
+    def _in_keys(self):
+        """The general path's input matrices, in the order of their rows in the one product."""
+        return ("q", "k") + (() if self.values_are_keys else ("v",)) + (("g",) if self.head_gate else ())
 
     def cache_need(self):
         if self.general:
@@ -139,20 +163,26 @@ class Attention(Part):
 
     def _load_general(self, tensors, build: BuildContext) -> None:
         nm, nh, nkv, dh, dv = self.names, self.heads, self.kv_heads, self.head_dim, self.value_dim
-        mats = [tensors[nm["q"]], tensors[nm["k"]], tensors[nm["v"]]] + ([tensors[nm["g"]]] if self.head_gate else [])
-        self.w_in = Weight(fused_rows(mats), build)
-        self.offsets = (0, nh * dh, (nh + nkv) * dh)
-        self.g_off = (nh + nkv) * dh + nkv * dv
+        self.w_in = Weight(fused_rows([tensors[nm[k]] for k in self._in_keys()]), build)
+        # (values that are the keys are read from the keys' columns of the product: the same numbers, before the norm)
+        self.offsets = (0, nh * dh, nh * dh if self.values_are_keys else (nh + nkv) * dh)
+        self.g_off = (nh + nkv) * dh + (0 if self.values_are_keys else nkv * dv)
         self.bias_vec = None
         if self.bias:       # one vector over the product's columns, 32-bit: added before anything is rounded
-            parts = [tensors[nm[k]].float() for k in ("q_bias", "k_bias", "v_bias")]
+            parts = [tensors[nm[k]].float() for k in ("q_bias", "k_bias") + (() if self.values_are_keys else ("v_bias",))]
             if self.head_gate:
                 parts.append(torch.zeros(nh, dtype=torch.float32, device=parts[0].device))
             self.bias_vec = torch.cat(parts).contiguous()
         self.q_head_norm = self.k_head_norm = None
-        if self.head_norm_eps is not None:
+        if self.head_norm_eps is not None and self.head_norm_weight:
             self.q_head_norm = tensors[nm["q_head_norm"]].float().contiguous()
             self.k_head_norm = tensors[nm["k_head_norm"]].float().contiguous()
+        elif self.head_norm_eps is not None:                  # a norm without a weight: the kernel multiplies by ones
+            self.q_head_norm = self.k_head_norm = torch.ones(dh, dtype=torch.float32, device=build.device)
+        if self.sink:
+            self.sinks = tensors[nm["sink"]].float().contiguous()
+        if self.out_bias:
+            self.output_bias = tensors[nm["o_bias"]].float().contiguous()
         self.page_size = build.page_size
         self.dtype = build.dtype
         # bfloat16: where a head size of the matrix-core kernels holds both the keys' and the values', both are stored
@@ -169,15 +199,20 @@ class Attention(Part):
                 ops.say_once(f"attention with {nh} heads of {dh} (values {dv}) in {nkv} groups runs on the generic kernel, not on the matrix cores")
         self.w_o = Weight(w_o.contiguous(), build)
         self.position.load({}, build)
-        if type(self.position).apply is not Part.apply or self.position.score_slopes() is not None:
-            raise ValueError("attention: the general path takes a rotation or no position encoding")
+        if type(self.position).apply is not Part.apply:
+            raise ValueError("attention: the general path takes a rotation, a bias inside the scores or no position encoding")
 
     def _matrix_cores(self, page_size: int) -> bool:
         """Whether the general path's attention runs on the matrix-core kernels (else on the generic one)."""
-        return (self.dtype == torch.bfloat16 and self.stored_value_dim == self.stored_dim
+        if self.position.score_slopes() is not None and not self.scale > 0:
+            return False
+        return (self.dtype == torch.bfloat16 and self.stored_value_dim == self.stored_dim and not self.sink
                 and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.stored_dim, page_size) is None)
 
-    def _forward_general(self, h, step, cache, out_dtype=None):
+    # forward(..., bias_later=True) leaves the output projection's bias (``output_bias``, float32, or None) to the caller
+    ends_in_bias = True
+
+    def _forward_general(self, h, step, cache, out_dtype=None, bias_later=False):
         nh, nkv = self.heads, self.kv_heads
         if not cache.writes:
             raise ops.KernelError("attention: the general path needs a cache of its own")
@@ -192,9 +227,12 @@ class Attention(Part):
         out = torch.empty((rows.shape[0], nh * self.stored_value_dim), dtype=self.dtype, device=rows.device)
         ops.paged_attention(q, out, cache.pages, step, cache.group, nh, nkv, self.stored_dim, page_size, self.scale,
                             self.window, value_dim=self.stored_value_dim, chunk=self.chunk,
-                            force_generic=not self._matrix_cores(page_size))
+                            force_generic=not self._matrix_cores(page_size), head_slopes=self.position.score_slopes(),
+                            sinks=self.sinks)
         if self.head_gate:
             ops.head_gate(out, rows, self.g_off, nh, self.stored_value_dim)
+        if self.output_bias is not None and not bias_later:
+            return ops.row_bias(linear(out, self.w_o, out_dtype=out_dtype or torch.float32), self.output_bias)
         return linear(out, self.w_o, out_dtype=out_dtype or self.dtype)
 
     def load(self, tensors, build: BuildContext) -> None:
@@ -239,7 +277,8 @@ class Attention(Part):
         page_size = self.own_page_size or self.page_size
         if self.general:
             if self._matrix_cores(page_size):
-                ops.plan_attention(step, self.heads, self.kv_heads, -self.chunk if self.chunk else self.window)
+                ops.plan_attention(step, self.heads, self.kv_heads, -self.chunk if self.chunk else self.window,
+                                   biased=self.position.score_slopes() is not None)
             return
         if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
                 and self.value_dim == self.padded_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.padded_dim, page_size) is None:
@@ -259,11 +298,11 @@ class Attention(Part):
             return False
         return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and skinny_takes(n_rows, self.w_qkv, preferred=True)
 
-    def forward(self, h, step, cache, into=None, planes_ok=False, out_dtype=None):
+    def forward(self, h, step, cache, into=None, planes_ok=False, out_dtype=None, bias_later=False):
         """``out_dtype``: the type of the branch's output if it is not the compute type (a block that adds
         several branches before the residual sum asks for float32)."""
         if self.general:
-            return self._forward_general(h, step, cache, out_dtype=out_dtype)
+            return self._forward_general(h, step, cache, out_dtype=out_dtype, bias_later=bias_later)
         nh, nkv, dh, dv = self.heads, self.kv_heads, self.padded_dim, self.value_dim       # (dh: as the kernels see a head)
         plain = self.norm_eps is None and self.q_temp is None       # nothing but a rotation between the product and the cache
         if not plain and self.position.rotary_tables() is not None:

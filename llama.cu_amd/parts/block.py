@@ -18,7 +18,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, NormedRows, Part, PartSpec, ScaledRows, SlotState, TensorSpec, make_part, prefixed, register_part
-from .norm import LayerNorm
+from .norm import LayerNorm, NoNorm
 
 
 class PreNormBlock(Part):
@@ -310,3 +310,75 @@ class SandwichBlock(Part):
 
 
 register_part("block", "sandwich", SandwichBlock)
+
+
+class PostNormBlock(Part):
+    """A norm behind every sublayer and none in front: ``x += post1(mixer(x))``, then ``x += post2(ffn(x))``; the sublayers
+    read the residual stream itself (rounded to the compute type).  The feed-forward, with its norm, may be missing.  The
+    norms are RMS norms (a factor per row times a weight per column).  The norm behind a sublayer, the residual sum and
+    the rounded copy of the new stream that the next sublayer reads are one kernel (``ops.norm_post``), also across the
+    border to the next block where that block takes such rows; a bias that the mixer's last product still lacks is
+    added in the same kernel.  The stream and the sums are 32-bit."""
+
+    def __init__(self, mixer: PartSpec, post1: PartSpec, ffn: Optional[PartSpec] = None, post2: Optional[PartSpec] = None):
+        if (ffn is None) != (post2 is None):
+            raise ValueError("post-norm block: the feed-forward and its norm come together or not at all")
+        self.specs = {"mixer": mixer, "post1": post1, "ffn": ffn, "post2": post2}
+        self.mixer = make_part("mixer", mixer)
+        self.post1 = make_part("norm", post1)
+        self.ffn = make_part("ffn", ffn) if ffn is not None else None
+        self.post2 = make_part("norm", post2) if post2 is not None else None
+        for name in ("post1", "post2"):
+            part = getattr(self, name)
+            if part is not None and (not part.deferrable or isinstance(part, NoNorm)):
+                raise ValueError(f"post-norm block: {name} must be a norm that is a factor per row times a weight per column")
+        self._reads = make_part("norm", PartSpec("none"))          # what stands where a first norm would
+        self.graph_safe = all(p.graph_safe for _, p in self._children())
+
+    tensors = SandwichBlock.tensors
+    fused_groups = SandwichBlock.fused_groups
+    cache_need = SandwichBlock.cache_need
+    prepare = SandwichBlock.prepare
+    decode_splits = SandwichBlock.decode_splits
+
+    def _children(self):
+        return [(self.specs[k].name, getattr(self, k)) for k in ("mixer", "post1", "ffn", "post2") if getattr(self, k) is not None]
+
+    def load(self, tensors, build: BuildContext) -> None:
+        SandwichBlock.load(self, tensors, build)
+        self._reads.load({}, build)
+
+    @property
+    def first_norm(self):
+        return self._reads
+
+    hands_over_normed = True     # forward(..., next_norm=) returns NormedRows
+    takes_normed_rows = True     # pending may be NormedRows made with first_norm (the rounded stream)
+
+    def _sum_and_read(self, x, a, post, a_bias, reader):
+        """``x += post(a + a_bias)`` and what ``reader`` (the next sublayer's norm, or none) makes of the new ``x``."""
+        if reader is None:
+            ops.norm_post(x, a, post.weight32, post.eps, a_bias=a_bias)
+            return None
+        if reader.weight32 is None:                  # no norm: the stream itself (a copy only where it is rounded)
+            if self.dtype == torch.float32:
+                ops.norm_post(x, a, post.weight32, post.eps, a_bias=a_bias)
+                return x
+            return ops.norm_post(x, a, post.weight32, post.eps, out_dtype=self.dtype, a_bias=a_bias, copy=True)
+        return ops.norm_post(x, a, post.weight32, post.eps, reader.weight32, reader.eps, out_dtype=self.dtype, a_bias=a_bias)
+
+    def forward(self, x: torch.Tensor, pending, step, cache, next_norm=None, planes_ok=False):
+        h = pending.rows if isinstance(pending, NormedRows) else self._reads.forward(x, pending)
+        later = bool(getattr(self.mixer, "ends_in_bias", False))
+        a = self.mixer.forward(h, step, cache, bias_later=True) if later else self.mixer.forward(h, step, cache)
+        last, post, bias = a, self.post1, (self.mixer.output_bias if later else None)
+        if self.ffn is not None:
+            h2 = self._sum_and_read(x, a, self.post1, bias, self._reads)
+            last, post, bias = self.ffn.forward(h2), self.post2, None
+        if next_norm is not None:
+            return NormedRows(self._sum_and_read(x, last, post, bias, next_norm))
+        self._sum_and_read(x, last, post, bias, None)
+        return None
+
+
+register_part("block", "post_norm", PostNormBlock)

@@ -1,4 +1,4 @@
-"""A feed-forward of many small experts of which every token uses a few.
+"""Feed-forwards of many small experts of which every token uses a few: ``SigmoidMoE`` (below) and ``GatedMoE`` (at the end).
 
     z = W_router h (32-bit),  s = sigmoid(z)
     the ``top`` experts with the largest scores are chosen (ties: the lower index), with s itself as weight (the weights of a token are not made to add up to one)
@@ -17,7 +17,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import fused_rows
-from .base import BuildContext, Part, TensorSpec, register_part
+from .base import BuildContext, Part, PartSpec, TensorSpec, make_part, register_part
 
 
 class SigmoidMoE(Part):
@@ -74,3 +74,87 @@ class SigmoidMoE(Part):
 
 
 register_part("ffn", "sigmoid_moe", SigmoidMoE)
+
+
+class GatedMoE(Part):
+    """Gated experts whose weights are a softmax over the chosen logits, with an optional shared expert.
+
+        z = W_router h + b (32-bit); the ``top`` largest are chosen (ties: the lower index); weights = softmax over the chosen z
+        out = sum over the chosen e of  weight_e * W_down[e] (silu(W_gate[e] h) * (W_up[e] h))
+              + sigmoid(w_sg . h) * shared(h)          (``shared``: a dense gated feed-forward that every token uses)
+
+    The weight scales what comes OUT of an expert.  The shared expert's gate is one more row of the router's matrix, so
+    its logit is made by the routing kernel, in 32-bit.  The output is 32-bit rows."""
+    graph_safe = True
+
+    NAMES = {"router": "router", "router_bias": "router.b", "gate": "e{}.gate", "up": "e{}.up", "down": "e{}.down",
+             "shared_gate": "shared.gate", "shared_up": "shared.up", "shared_down": "shared.down", "shared_sg": "shared.sg"}
+
+    def __init__(self, hidden_size: int, expert_size: int, experts: int, top: int, shared_size: Optional[int] = None,
+                 router_bias: bool = True, names: Optional[Dict[str, str]] = None):
+        self.hidden_size, self.expert_size = int(hidden_size), int(expert_size)
+        self.experts, self.top = int(experts), int(top)
+        if not 1 <= self.top <= self.experts or self.experts > 1024:
+            raise ValueError(f"moe: top {top} of {experts} experts is not supported (1 <= top <= experts <= 1024)")
+        self.names = dict(self.NAMES, **(names or {}))
+        self.router_bias = bool(router_bias)
+        self.shared = None
+        if shared_size is not None:
+            nm = self.names
+            self.shared = make_part("ffn", PartSpec("swiglu", {"hidden_size": self.hidden_size, "intermediate_size": int(shared_size),
+                                                               "names": {"gate": nm["shared_gate"], "up": nm["shared_up"],
+                                                                         "down": nm["shared_down"]}}))
+            self.graph_safe = self.shared.graph_safe
+
+    def _each(self, key):
+        return [self.names[key].format(e) for e in range(self.experts)]
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        d, ff, nm = self.hidden_size, self.expert_size, self.names
+        t = {nm["router"]: TensorSpec((self.experts, d))}
+        if self.router_bias:
+            t[nm["router_bias"]] = TensorSpec((self.experts,))
+        for key, shape in (("gate", (ff, d)), ("up", (ff, d)), ("down", (d, ff))):
+            for n in self._each(key):
+                t[n] = TensorSpec(shape)
+        if self.shared is not None:
+            t.update(self.shared.tensors())
+            t[nm["shared_sg"]] = TensorSpec((1, d))
+        return t
+
+    def fused_groups(self, dtype, device):
+        groups = [(tuple(self._each(k)), 0) for k in ("gate", "up", "down")]
+        return groups + (self.shared.fused_groups(dtype, device) if self.shared is not None else [])
+
+    def load(self, tensors, build: BuildContext) -> None:
+        d, ff, n, nm = self.hidden_size, self.expert_size, self.experts, self.names
+        rows = [tensors[nm["router"]].float()] + ([tensors[nm["shared_sg"]].float().view(1, d)] if self.shared is not None else [])
+        self.router = torch.cat(rows).contiguous()                          # the router, and the shared expert's gate, are 32-bit
+        self.bias = tensors[nm["router_bias"]].float().contiguous() if self.router_bias else None
+        gate = fused_rows([tensors[k] for k in self._each("gate")]).view(n, ff, d)
+        up = fused_rows([tensors[k] for k in self._each("up")]).view(n, ff, d)
+        self.w_down = fused_rows([tensors[k] for k in self._each("down")]).view(n, d, ff)
+        if ff % 16:
+            # the products take an expert's features 16 at a time: rows of zeros in gate and up and the columns of zeros
+            # that meet them in the down matrix change nothing (silu(0) * 0 = 0)
+            pad = 16 - ff % 16
+            gate = torch.cat([gate, gate.new_zeros(n, pad, d)], dim=1)
+            up = torch.cat([up, up.new_zeros(n, pad, d)], dim=1)
+            self.w_down = torch.cat([self.w_down, self.w_down.new_zeros(n, d, pad)], dim=2).contiguous()
+        self.w_gate_up = ops.gated_rows(gate.contiguous(), up.contiguous())
+        if self.shared is not None:
+            self.shared.load(tensors, build)
+        self.dtype = build.dtype
+
+    def forward(self, h):
+        routed = ops.moe_route(h, self.router, self.top, bias=self.bias, softmax_chosen=True, extra=1 if self.shared is not None else 0)
+        ids, wts = routed[0], routed[1]
+        out = torch.zeros((h.shape[0], self.hidden_size), dtype=torch.float32, device=h.device)
+        if self.shared is not None:
+            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True, shared=self.shared.forward(h), shared_gate=routed[2])
+        else:
+            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True)
+        return out
+
+
+register_part("ffn", "gated_moe", GatedMoE)

@@ -82,5 +82,27 @@ class LayerNorm(Part):
         return ops.layernorm(x, self.weight, self.bias, self.eps, out, delta=delta)
 
 
+class NoNorm(Part):
+    """No normalisation at all: the rows of the residual stream themselves, rounded to the compute type, for a sublayer
+    that reads the stream as it is.  It stands where a block's first norm would, so that whoever adds the last output
+    before it may hand the rounded rows over (``weight32`` None tells ``ops.norm_post`` to copy)."""
+    graph_safe = True
+    deferrable = True
+    weight = weight32 = None
+
+    def __init__(self, size: int = 0):
+        self.size, self.eps = int(size), 0.0
+        self.dtype = None
+
+    def load(self, tensors, build: BuildContext) -> None:
+        self.dtype = build.dtype
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if delta is not None:
+            ops.residual_add(x, delta)
+        return x if self.dtype == torch.float32 else x.to(self.dtype)
+
+
+register_part("norm", "none", NoNorm)
 register_part("norm", "rmsnorm", RMSNorm)
 register_part("norm", "layernorm", LayerNorm)
