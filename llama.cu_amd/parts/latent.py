@@ -85,12 +85,13 @@ class LatentAttention(Part):
         self.w_o = Weight(tensors[nm["o"]], build)
         self.position.load({}, build)
         if build.dtype == torch.bfloat16:
-            # where a head size of the matrix-core kernels holds [c, r], key and value are both stored at that size
+            # where a head size of the matrix-core kernels holds [c, r], key and value are both stored at that size (whatever
+            # the layer's heads: a layer that reads this cache may have other heads, and must find the same sizes)
             for size in (32, 64, 96, 128):
-                if size >= rank + self.rot_dim and ops.mfma_attention_refusal(build.dtype, nh, 1, size, self.own_page_size or build.page_size) is None:
+                if size >= rank + self.rot_dim and ops.mfma_attention_refusal(build.dtype, 1, 1, size, self.own_page_size or build.page_size) is None:
                     self.stored_dim = self.stored_value_dim = size
                     break
-            else:
+            if not self._matrix_cores(self.own_page_size or build.page_size):
                 ops.say_once(f"latent attention with {nh} heads over a latent of {rank} + {self.rot_dim} runs on the generic kernel, not on the matrix cores")
 
     def _matrix_cores(self, page_size: int) -> bool:
