@@ -100,8 +100,16 @@ def sharpened(cfg: dict, factor: float) -> dict:
     return out
 
 
-def random_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
-    """Every tensor of the design for ``cfg``, float32 values that bfloat16 holds exactly."""
+TAGS = 4        # channels of the stream that a steady router reads
+
+
+def random_weights(cfg: dict, seed: int, steady_router: bool = False) -> Dict[str, torch.Tensor]:
+    """Every tensor of the design for ``cfg``, float32 values that bfloat16 holds exactly.  ``steady_router``: for runs in
+    bfloat16, whose stream differs from the plain model's by some hundredths, which would make close calls between
+    experts fall the other way (a choice is discrete; such a flip moves the logits by their size and is no fault): the
+    first ``TAGS`` channels of the embedding hold small integers, no norm behind a sublayer writes into them (weights of
+    zero there), and the routers read these channels alone, so that the routers' logits are the same numbers in every
+    run while the choice still differs from token to token and from layer to layer."""
     g = torch.Generator().manual_seed(seed)
     d = cfg["width"]
 
@@ -111,10 +119,17 @@ def random_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
     def vec(n, mean=0.0, std=0.1):
         return mean + std * torch.randn(n, generator=g)
 
+    def steady(norm_weight):
+        if steady_router:
+            norm_weight[:TAGS] = 0.0
+        return norm_weight
+
     w = {"embed": torch.randn(cfg["vocab"], d, generator=g), "final.norm": vec(d, 1.0), "head": mat(cfg["vocab"], d)}
+    if steady_router:
+        w["embed"][:, :TAGS] = torch.randint(-3, 4, (cfg["vocab"], TAGS), generator=g).float()
     for i, layer in enumerate(cfg["layers"]):
         pre, m = f"l{i}.mix.", layer["mixer"]
-        w[f"l{i}.norm1"] = vec(d, 1.0, 0.2)
+        w[f"l{i}.norm1"] = steady(vec(d, 1.0, 0.2))
         if layer["type"] == "attention":
             w[pre + "q"], w[pre + "q.b"] = mat(m["heads"] * m["dim"], d), vec(m["heads"] * m["dim"], std=0.3)
             w[pre + "k"], w[pre + "k.b"] = mat(m["kv_heads"] * m["dim"], d), vec(m["kv_heads"] * m["dim"], std=0.3)
@@ -130,7 +145,7 @@ def random_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
         f = layer.get("mlp")
         if f is None:
             continue
-        w[f"l{i}.norm2"] = vec(d, 1.0, 0.2)
+        w[f"l{i}.norm2"] = steady(vec(d, 1.0, 0.2))
         pre = f"l{i}.mlp."
         if f["kind"] == "dense":
             w[pre + "gate"], w[pre + "up"], w[pre + "down"] = mat(f["ff"], d), mat(f["ff"], d), mat(d, f["ff"])
@@ -140,6 +155,9 @@ def random_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
             w[f"{pre}e{e}.gate"], w[f"{pre}e{e}.up"], w[f"{pre}e{e}.down"] = mat(ff, d), mat(ff, d, 2.0), mat(d, ff, 2.0)
         # logits well apart: a choice between experts is discrete, and a close call may fall the other way under rounding
         w[pre + "router"], w[pre + "router.b"] = mat(f["router"]["experts"], d, 3.0), vec(f["router"]["experts"], std=1.0)
+        if steady_router:
+            w[pre + "router"][:, TAGS:] = 0.0
+            w[pre + "router"][:, :TAGS] = torch.randint(-4, 5, (f["router"]["experts"], TAGS), generator=g).float() / 4
         if f.get("shared") is not None:
             sf = f["shared"]["ff"]
             w[pre + "shared.gate"], w[pre + "shared.up"], w[pre + "shared.down"] = mat(sf, d), mat(sf, d), mat(d, sf)

@@ -13,7 +13,7 @@ import torch
 
 import plain_ralepel as P
 from ralepel_common import (CONFIGS, as_numpy, assert_close, attention, config, dense, latent, make_folder, moe, plain_logits,
-                            random_weights, safe_tokens, sharpened, tokens_of)
+                            random_weights, sharpened, tokens_of)
 
 pytestmark = pytest.mark.gpu
 TYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
@@ -219,7 +219,7 @@ def test_latent_attention_and_a_layer_that_reads_its_latent(dtype, nh, dn, dr, d
     got, again = feed.run(forward, [torch.cat([a, b], dim=1) for a, b in zip(rows, rows2)])
     n1 = {"a." + k: v.double().numpy() for k, v in w1.items()}
     n2 = {"b." + k: v.double().numpy() for k, v in w2.items()}
-    tol = 2e-4 if dtype == "float32" else 4e-2
+    tol = 2e-4 if dtype == "float32" else REL["bfloat16"]      # (the folded form rounds the folded queries and the mixed latents once more)
     for r in range(2):
         pair = P.latent_pair(rows[r].double().numpy(), m1, n1, "a.", eps)
         assert_close(got[r][:, :d], P.latent_attention(rows[r].double().numpy(), m1, n1, "a.", pair), tol, f"request {r}")
@@ -292,12 +292,14 @@ def test_ties_between_experts_go_to_the_lower_index():
 _made = {}
 
 
-def model(name, sharp=1.0):
-    """(configuration, weights, folder) of a test model, made once."""
-    key = (name, sharp)
+def model(name, sharp=1.0, dtype="float32"):
+    """(configuration, weights, folder) of a test model, made once.  For runs in bfloat16 the routers are steady ones
+    (``random_weights``): their logits do not feel the rounding of the stream, so that no choice of experts is a close call
+    that falls differently in two runs; the runs in float32 have routers that read the whole stream."""
+    key = (name, sharp, dtype == "bfloat16")
     if key not in _made:
         cfg = sharpened(CONFIGS[name], sharp) if sharp != 1.0 else CONFIGS[name]
-        w = random_weights(cfg, 1 + sorted(CONFIGS).index(name))
+        w = random_weights(cfg, 1 + sorted(CONFIGS).index(name), steady_router=key[2])
         _made[key] = (cfg, w, make_folder(cfg, w))
     return _made[key]
 
@@ -312,9 +314,8 @@ def runner_for(folder, dtype, **kw):
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"), ("C", "float32"),
                                         ("C", "bfloat16"), ("D", "float32"), ("E", "float32")])
 def test_a_whole_prompt_against_the_plain_model(name, dtype):
-    cfg, w, folder = model(name)
-    # (a choice of experts is discrete: in bfloat16 only sequences without a close call are compared with the plain model)
-    toks = tokens_of(cfg["vocab"], 100, 1) if dtype == "float32" else safe_tokens(cfg, w, 40, 1)
+    cfg, w, folder = model(name, dtype=dtype)
+    toks = tokens_of(cfg["vocab"], 100, 1)
     want = plain_logits(cfg, w, toks)
     r = runner_for(folder, dtype, page_size={"A": 16, "B": 32, "C": 48, "D": 64, "E": 16}[name])
     got = r.step([0], [toks], [list(range(len(toks)))])
@@ -327,8 +328,8 @@ def test_a_whole_prompt_against_the_plain_model(name, dtype):
 def test_models_of_one_kind_of_mixer_and_the_first_tokens_of_a_sequence(name, dtype):
     """Latent layers alone (one pool, no window) and windowed layers alone: a prompt in portions, then tokens one by one,
     a second request beside the first that starts with portions of one and two tokens, pages used again."""
-    cfg, w, folder = model(name)
-    a, b = safe_tokens(cfg, w, 40, 50), safe_tokens(cfg, w, 21, 51)
+    cfg, w, folder = model(name, dtype=dtype)
+    a, b = tokens_of(cfg["vocab"], 40, 50), tokens_of(cfg["vocab"], 21, 51)
     wa, wb = plain_logits(cfg, w, a), plain_logits(cfg, w, b)
     r = runner_for(folder, dtype, max_seqs=2, max_tokens=128)
     got_a = [r.step([0], [a[:17]], [list(range(17))]).clone()]
@@ -349,12 +350,11 @@ def test_models_of_one_kind_of_mixer_and_the_first_tokens_of_a_sequence(name, dt
 
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "float32")])
 def test_prefill_against_token_by_token_decoding_and_portions_down_to_two_tokens(name, dtype):
-    cfg, w, folder = model(name)
+    cfg, w, folder = model(name, dtype=dtype)
     toks = tokens_of(cfg["vocab"], 90, 2)
     r = runner_for(folder, dtype)
     whole = r.step([0], [toks], [list(range(len(toks)))]).clone()
-    if dtype == "float32":
-        assert_close(whole, plain_logits(cfg, w, toks), REL[dtype], "the whole prompt")
+    assert_close(whole, plain_logits(cfg, w, toks), REL[dtype], "the whole prompt")
     # one token at a time from the first (long enough for captured graphs to replay)
     single = torch.cat([r.step([1], [[t]], [[0]]).clone() for t in toks])
     sizes, at, parts = [2, 3, 5, 1, 17, 2, 31, 4, 2, 1, 64], 0, []
@@ -379,7 +379,8 @@ def test_batches_of_unequal_requests_and_pages_used_again(name, dtype):
     """Seven requests of unequal lengths through an engine with three slots and a pool that holds only what is live:
     portions of some beside single tokens of others; finished requests give their pages to new ones (pages that
     change hands are filled with NaN first).  Every request's logits equal those it gets alone."""
-    cfg, w, folder = model(name, sharp=3.0)
+    # (peaked scores multiply what the rounding of queries and keys does to a softmax's weights: less peaked in bfloat16)
+    cfg, w, folder = model(name, sharp=3.0 if dtype == "float32" else 1.5, dtype=dtype)
     lens = [70, 33, 1, 48, 19, 90, 7]
     reqs = [tokens_of(cfg["vocab"], n, 10 + i) for i, n in enumerate(lens)]
     r = runner_for(folder, dtype, max_seqs=3, max_tokens=3 * 96, max_batch_tokens=256, poison_freed=True)
@@ -438,14 +439,13 @@ def test_keys_far_back_at_page_borders_and_at_the_edges_of_windows(name):
 
 
 def test_long_decoding_in_bfloat16():
-    cfg, w, folder = model("B")
+    cfg, w, folder = model("B", dtype="bfloat16")
     toks = tokens_of(cfg["vocab"], 260, 8)
     r = runner_for(folder, "bfloat16")
     want = r.step([1], [toks], [list(range(260))]).clone()
     got = [r.step([0], [toks[:20]], [list(range(20))]).clone()] + [r.step([0], [[t]], [[0]]).clone() for t in toks[20:]]
-    # (a close call between experts may fall the other way in one of the two runs: a few positions may differ by more)
-    err = (torch.cat(got) - want).abs().amax(dim=1) / want.abs().max()
-    assert (err <= SAME["bfloat16"]).float().mean() >= 0.97 and torch.isfinite(err).all(), f"long decoding against the whole prompt: {err.max():.3e}"
+    assert_close(torch.cat(got), want, SAME["bfloat16"], "long decoding against the whole prompt")
+    assert_close(want, plain_logits(cfg, w, toks), REL["bfloat16"], "the whole prompt against the plain model")
     assert sum(r.graph_replays.values()) > 100, "decoding was not replayed from captured graphs"
 
 
@@ -465,7 +465,7 @@ def test_greedy_generation_through_the_engine_and_its_scheduler(dtype):
     """The framework's entry point: prompts of unequal lengths, more than run at a time, prefilled in portions; the
     generated tokens equal the plain model's arg-max continuation."""
     from llama_cu_amd.engine.engine import Engine
-    cfg, w, folder = model("B")
+    cfg, w, folder = model("B", dtype=dtype)
     prompts = [tokens_of(cfg["vocab"], n, 30 + i) for i, n in enumerate([21, 5, 40, 2, 13])]
     steps = 12
     engine = Engine.from_folder(folder, dtype=dtype, page_size=16, max_tokens=512, max_seqs=3, prefill_chunk=16)
