@@ -389,8 +389,36 @@ def lozezen_config(z, positions):
                                     "embedding": {"scale": 2.0}, "max_positions": positions})
 
 
+def ralepel_config(z, positions):
+    """Attention with a sink within a window of 1,024 and latent attention in turn (every second latent layer reads the
+    latent of the one before it); the first layer with the dense feed-forward of the Llama model beside it, the others
+    with a mixture of experts whose active weights (the chosen experts and the shared one) are about as many.  The latent
+    and its rotated part are 96 + 32 dims: one head of the matrix-core attention kernels' largest size."""
+    from llama_cu_amd.config import RalepelConfig
+    inter = (z["top"] * 2 * z["ff"] // 3 + 127) // 128 * 128
+    shared = inter // 4 // 64 * 64
+    expert = (inter - shared) // z["top"] // 64 * 64
+    d, h, g, w = z["dim"], z["heads"], z["kv_heads"], z["width"]
+    layers, last_latent = [], None
+    for i in range(z["layers"]):
+        if i % 2 == 0:
+            kind, m = "attention", {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024}}
+        else:
+            kind, m = "latent_attention", {"heads": h, "dim": 96, "rot_dim": 32, "vdim": d, "kv_rank": 96, "scale": d ** -0.5,
+                                           "rot": {"dims": 32, "base": 50000.0}}
+            if i % 4 == 3 and last_latent is not None:
+                m["kv_from"] = last_latent
+            else:
+                last_latent = i
+        mlp = {"kind": "dense", "ff": inter} if i == 0 else \
+            {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"]}, "expert": {"ff": expert}, "shared": {"ff": shared}}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    return RalepelConfig.from_dict({"architecture": "Ralepel", "vocab": z["vocab"], "width": w, "layers": layers, "norm": {"eps": 1e-5},
+                                    "max_positions": positions})
+
+
 DESIGN_CONFIGS = {"divasun": lambda z, p: divasun_config(z, p), "llama": lambda z, p: llama_like(z, p),
-                  "lozezen": lambda z, p: lozezen_config(z, p)}
+                  "lozezen": lambda z, p: lozezen_config(z, p), "ralepel": lambda z, p: ralepel_config(z, p)}
 
 
 def llama_like(z, positions):
@@ -517,10 +545,10 @@ def main() -> int:
                          "decode while a prompt of 16 tokens arrives every second step (host time and the GPU's busy "
                          "fraction per kind of step)")
     ap.add_argument("--designs", default="divasun,llama", metavar="NAMES",
-                    help="with --workload designs: which designs are measured side by side, of divasun, lozezen and llama "
+                    help="with --workload designs: which designs are measured side by side, of divasun, lozezen, ralepel and llama "
                          "(default: divasun,llama)")
     ap.add_argument("--designs-one", metavar="DESIGN:SIZE:WHAT", default=None,
-                    help="with --workload designs, for a profiler: only DESIGN (divasun, lozezen or llama) at SIZE (w2048, w4096), and "
+                    help="with --workload designs, for a profiler: only DESIGN (divasun, lozezen, ralepel or llama) at SIZE (w2048, w4096), and "
                          "only WHAT: 'prefill' (three steps of 2,048 tokens) or a number of requests that decode ten steps over "
                          "prompts of 512 tokens; steps are launched one kernel at a time, not replayed from graphs")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64, the prefill and the check")

@@ -57,12 +57,24 @@ __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
 // point takes head_slopes [nh] as well, and slope[h] * (j - p) is added to the scaled score of key j for the query at
 // position p of head h (a bias that grows with the distance).  Inside the kernels the bias stands in the scores' own
 // units (slope / scale), so that everything after the scores is the same code.
+// The same library takes sinks [nh] (may be null) behind the slopes: exp(sink[h]) stands in the denominator of every
+// softmax of head h beside the keys' terms, with no key, value, scale or bias.  It enters where a row's sum is
+// final (sink_share below): once, also where a request's keys were walked in parts.
 #ifdef LCU_SCORE_BIAS
-#define BIAS_KPARAMS , const float *__restrict__ head_slopes, float inv_scale
-#define BIAS_KARGS(scale) , head_slopes, 1.0f / (scale)
-#define BIAS_PARAMS , const float *head_slopes
-#define BIAS_ARGS , head_slopes
+#define BIAS_KPARAMS , const float *__restrict__ head_slopes, float inv_scale, const float *__restrict__ sinks
+#define BIAS_KARGS(scale) , head_slopes, 1.0f / (scale), sinks
+#define BIAS_PARAMS , const float *head_slopes, const float *sinks
+#define BIAS_ARGS , head_slopes, sinks
+#define MERGE_SINKS sinks
+// A row whose keys gave the sum l of 2^(score - m) takes in its sink: returns the factor for the row's
+// unnormalised output, 2^(m - m') / (l 2^(m - m') + 2^(sink log2(e) - m')) with m' = max(m, sink log2(e)).
+__device__ __forceinline__ float sink_share(float m, float l, float sink) {
+    const float sk = sink * 1.4426950408889634f, m_all = fmaxf(m, sk);
+    const float keep = exp2f(m - m_all);                 // (m = -inf, no key at all: 0)
+    return keep / (l * keep + exp2f(sk - m_all));
+}
 #else
+#define MERGE_SINKS nullptr
 #define BIAS_KPARAMS
 #define BIAS_KARGS(scale)
 #define BIAS_PARAMS
@@ -417,6 +429,12 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
         }
         const int head = head0 + row;
         if (n_splits == 1) {
+#ifdef LCU_SCORE_BIAS
+            if (sinks) {
+                out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val * sink_share(M_safe, L, sinks[head]));
+                continue;
+            }
+#endif
             out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val / L);
         } else {
             const size_t slot = ((size_t)ri * nh + head) * n_splits + split;
@@ -434,7 +452,7 @@ template <int DH>
 __global__ void __launch_bounds__(DH / 4)
 attention_merge_kernel(bf16_t *__restrict__ out, int out_stride, const float *__restrict__ part_o,
                        const float *__restrict__ part_ml, const int *__restrict__ q_start,
-                       const int *__restrict__ req_list, int nh, int n_splits) {
+                       const int *__restrict__ req_list, int nh, int n_splits, const float *__restrict__ sinks) {
     // a thread has four dims of one (token, head); the loads of up to eight parts are issued
     // together, so the kernel takes one trip to memory and not one per part
     constexpr int GROUP = 8;
@@ -468,7 +486,10 @@ attention_merge_kernel(bf16_t *__restrict__ out, int out_stride, const float *__
         }
         M = Mn;
     }
-    const float inv = 1.0f / L;
+    float inv = 1.0f / L;
+#ifdef LCU_SCORE_BIAS
+    if (sinks) inv = sink_share(M == -INFINITY ? 0.f : M, L, sinks[head]);
+#endif
     u32x2 w;
     w.x = pack_bf16(acc[0] * inv, acc[1] * inv);
     w.y = pack_bf16(acc[2] * inv, acc[3] * inv);
@@ -497,7 +518,7 @@ static int launch_decode(const void *q, int q_stride, void *out, int out_stride,
     LCU_LAUNCH_CHECK();
     if (n_splits > 1) {
         attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(DH / 4), 0, stream>>>((bf16_t *)out, out_stride, part_o, part_ml,
-                                                                                q_start, req_list, nh, n_splits);
+                                                                                q_start, req_list, nh, n_splits, MERGE_SINKS);
         LCU_LAUNCH_CHECK();
     }
     return LCU_OK;
@@ -1077,7 +1098,10 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     // ---- a row's sum lies in its two lanes (each added the keys it held); the output is written as it stands
     float l_all = st.l;
     l_all += __shfl_xor(l_all, 32, WAVE);
-    const float inv = 1.0f / l_all;
+    float inv = 1.0f / l_all;
+#ifdef LCU_SCORE_BIAS
+    if (sinks && tok_row >= 0) inv = sink_share(st.m, l_all, sinks[head0 + n % hc]);
+#endif
     if (tok_row >= 0) {
         bf16_t *o = out + (size_t)tok_row * out_stride + (size_t)(head0 + n % hc) * DH;
 #pragma unroll

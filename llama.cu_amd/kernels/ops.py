@@ -391,7 +391,7 @@ def mfma_attention_supported(q: torch.Tensor, n_heads: int, n_kv_heads: int, hea
 
 def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_heads, n_kv_heads, head_dim, page_size,
                      scale, window, n_splits, req_list: Optional[torch.Tensor] = None,
-                     head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     head_slopes: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Matrix-core attention for requests that feed one token each: all ``n_req`` requests of
     the batch, or the ``n_req`` whose indices ``req_list`` holds.  ``head_slopes``: the bias on the distance inside
     the scores (the kernels of the second library, ``attention_mfma_bias``)."""
@@ -402,7 +402,7 @@ def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_head
         part_o = torch.empty(n_req * n_heads * n_splits * head_dim, dtype=torch.float32, device=q.device)
         part_ml = torch.empty(n_req * n_heads * n_splits * 2, dtype=torch.float32, device=q.device)
     lib = build.load("attention_mfma" if head_slopes is None else "attention_mfma_bias")
-    more = () if head_slopes is None else (_ptr(head_slopes),)
+    more = () if head_slopes is None else (_ptr(head_slopes), _ptr(sinks))
     _check(lib.lcu_attention_decode_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(block_table),
                                          block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(req_list), n_req, n_heads,
                                          n_kv_heads,
@@ -449,7 +449,7 @@ def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: b
 
 def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, n_heads,
                       n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev: Optional[torch.Tensor] = None,
-                      head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      head_slopes: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Matrix-core attention for any mix of portions and single tokens.  ``n_tasks_dev`` (int32 on the device, one
     entry): the lists hold that many tasks, at most ``n_tasks``, for which the grid is made."""
     if task_req.numel() < n_tasks or task_tok0.numel() < n_tasks:
@@ -459,7 +459,7 @@ def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, ta
         _gpu(n_tasks_dev)
         _i32(n_tasks_dev, "n_tasks_dev")
     lib = build.load("attention_mfma" if head_slopes is None else "attention_mfma_bias")
-    more = () if head_slopes is None else (_ptr(head_slopes),)
+    more = () if head_slopes is None else (_ptr(head_slopes), _ptr(sinks))
     _check(lib.lcu_attention_prefill_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache),
                                           ctypes.c_longlong(cache.shape[0]), _ptr(block_table),
                                           block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(task_req),
@@ -560,6 +560,16 @@ def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -
     return 1 + next(i for i, f in enumerate(fill) if f >= max(fill) - t.decode_fill_slack)
 
 
+_zeros: Dict = {}
+
+
+def _zero_slopes(n_heads: int, device) -> torch.Tensor:
+    key = (n_heads, str(device))
+    if key not in _zeros:
+        _zeros[key] = torch.zeros(n_heads, dtype=torch.float32, device=device)
+    return _zeros[key]
+
+
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
                     n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0,
                     force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0,
@@ -567,15 +577,21 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
     ``group``: picks the kernel for the batch's shape and type.  ``chunk``: keys of the query's own chunk of so many
     positions only (the matrix-core kernels take it as a negative window).  With a bias inside the scores
-    (``head_slopes``) the matrix-core kernels are those of the second library, which need a positive scale."""
+    (``head_slopes``) or with ``sinks`` (``exp(sink[h])`` in the denominator of head ``h``'s softmax) the matrix-core
+    kernels are those of the second library, which need a positive scale."""
     bt = step.block_table(group)
+    if sinks is not None:
+        _gpu(sinks)
+        if sinks.dtype != torch.float32 or sinks.shape != (n_heads,) or not sinks.is_contiguous():
+            raise KernelError(f"attention: sinks must be contiguous float32 [{n_heads}]")
     if head_slopes is not None:
         _gpu(head_slopes)
         if head_slopes.dtype != torch.float32 or head_slopes.shape != (n_heads,) or not head_slopes.is_contiguous():
             raise KernelError(f"attention: head_slopes must be contiguous float32 [{n_heads}]")
     if chunk and window:
         raise KernelError("attention: a window and chunks together are not supported")
-    if force_generic or sinks is not None or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
+    second = head_slopes is not None or sinks is not None          # the library with the bias and the sinks
+    if force_generic or (second and not scale > 0) or (value_dim and value_dim != head_dim) \
             or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
         return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
                                        n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim, chunk, sinks)
@@ -583,22 +599,24 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                         page_size)
     if chunk:
         window = -int(chunk)
+    if sinks is not None and head_slopes is None:
+        head_slopes = _zero_slopes(n_heads, q.device)              # sinks without a bias: slopes of zero
     if step.decode_only:
         splits = step.attn_splits or decode_splits(step.n_req, n_heads, n_kv_heads, step.max_ctx_len)
         # the workgroups start in the order of the requests' list: the requests with the most keys first, where the
         # batch says which they are (64 requests of 150 to 2,200 keys: the step 11.2 -> 11.0 ms)
         return attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, step.n_req, n_heads, n_kv_heads, head_dim,
-                                page_size, scale, window, splits, req_list=step.decode_order, head_slopes=head_slopes)
+                                page_size, scale, window, splits, req_list=step.decode_order, head_slopes=head_slopes, sinks=sinks)
     # a mixed batch: the requests that decode one token go to the decode kernel, the portions
     # to the prefill kernel (each would be slow at the other's work)
-    plan = plan_attention(step, n_heads, n_kv_heads, window, biased=head_slopes is not None)
+    plan = plan_attention(step, n_heads, n_kv_heads, window, biased=second)
     if plan.n_single:
         attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, plan.n_single, n_heads, n_kv_heads, head_dim, page_size,
-                         scale, window, plan.single_splits, req_list=plan.singles, head_slopes=head_slopes)
+                         scale, window, plan.single_splits, req_list=plan.singles, head_slopes=head_slopes, sinks=sinks)
     if plan.max_tasks:
         attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, plan.task_req, plan.task_tok0, plan.max_tasks,
                           plan.per_wg, n_heads, n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev=plan.n_tasks_dev,
-                          head_slopes=head_slopes)
+                          head_slopes=head_slopes, sinks=sinks)
     return out
 
 

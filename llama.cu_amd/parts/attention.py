@@ -204,9 +204,9 @@ class Attention(Part):
 
     def _matrix_cores(self, page_size: int) -> bool:
         """Whether the general path's attention runs on the matrix-core kernels (else on the generic one)."""
-        if self.position.score_slopes() is not None and not self.scale > 0:
+        if (self.position.score_slopes() is not None or self.sink) and not self.scale > 0:
             return False
-        return (self.dtype == torch.bfloat16 and self.stored_value_dim == self.stored_dim and not self.sink
+        return (self.dtype == torch.bfloat16 and self.stored_value_dim == self.stored_dim
                 and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.stored_dim, page_size) is None)
 
     # forward(..., bias_later=True) leaves the output projection's bias (``output_bias``, float32, or None) to the caller
@@ -278,7 +278,7 @@ class Attention(Part):
         if self.general:
             if self._matrix_cores(page_size):
                 ops.plan_attention(step, self.heads, self.kv_heads, -self.chunk if self.chunk else self.window,
-                                   biased=self.position.score_slopes() is not None)
+                                   biased=self.position.score_slopes() is not None or self.sink)
             return
         if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
                 and self.value_dim == self.padded_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.padded_dim, page_size) is None:
