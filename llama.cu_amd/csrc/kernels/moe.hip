@@ -399,14 +399,15 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
     }
 }
 
-// out[t, c] += sum_k wts[t, k] * y[t * top + k, c]  (in the order of k; wts null: ones)  + gate[t] * shared[t, c]  (shared null: nothing)
+// out[t, c] (+)= sum_k wts[t, k] * y[t * top + k, c]  (in the order of k; wts null: ones)  + gate[t] * shared[t, c]  (shared null: nothing)
+// fresh: out is written, not added to (what it held is not read).
 template <class T>
 __global__ void moe_combine_kernel(float *__restrict__ out, const float *__restrict__ y, const float *__restrict__ wts,
-                                   const T *__restrict__ shared, const float *__restrict__ gate, int n, int d, int top) {
+                                   const T *__restrict__ shared, const float *__restrict__ gate, int n, int d, int top, int fresh) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= d) return;
     for (size_t t = blockIdx.y; t < (size_t)n; t += gridDim.y) {
-        float acc = out[t * d + c];
+        float acc = fresh ? 0.f : out[t * d + c];
         for (int k = 0; k < top; ++k) acc += (wts ? wts[t * top + k] : 1.f) * y[(t * top + k) * d + c];
         if (shared) acc += (gate ? gate[t] : 1.f) * to_f32(shared[t * d + c]);
         out[t * d + c] = acc;
@@ -441,15 +442,17 @@ LCU_API int lcu_moe_route(const void *h, int type, const float *router, const fl
 // w_up: [experts, ff, d], w_down: [experts, d, ff] of `type`.  act: scratch [total, ff] of `type`; y: scratch
 // [total, d] 32-bit (only read and written when top > 1 or gated).  out: [n, d] 32-bit, added to.
 // gated: w_up is [experts, 2 * ff, d], in turns 16 rows of the gate matrix and the 16 rows of the up matrix that meet
-// them (ff a multiple of 16); act = silu(gate h) * (up h), and the weight scales what comes out.  shared (null or
+// them (ff a multiple of 16); act = silu(gate h) * (up h), and the weight scales what comes out; fresh: out is written
+// and not added to.  shared (null or
 // [n, d] of `type`) with shared_gate (null or [n] 32-bit): rows that are added beside the experts', times the gate.
 LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float *wts, int *ints, int max_tiles,
                             const void *w_up, const void *w_down, void *act, float *y, float *out, int n, int d, int ff,
-                            int experts, int top, int gated, const void *shared, const float *shared_gate, hipStream_t stream) {
+                            int experts, int top, int gated, const void *shared, const float *shared_gate, int fresh,
+                            hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     const int per = type == LCU_BF16 ? 8 : 4;
     if (d <= 0 || ff <= 0 || d % per || ff % per || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || max_tiles <= 0 ||
-        (type != LCU_F32 && type != LCU_BF16) || (gated && ff % 16) || (shared && !gated))
+        (type != LCU_F32 && type != LCU_BF16) || (gated && ff % 16) || (shared && !gated) || (fresh && !gated))
         return LCU_BAD_ARGUMENT;
     const int total = n * top;
     const int tile_rows = lcu_moe_tile_rows(total, experts);
@@ -484,8 +487,8 @@ LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float
     LCU_LAUNCH_CHECK();
     if (!add) {
         const dim3 gc((d + 255) / 256, n < 65535 ? n : 65535);
-        if (type == LCU_BF16) moe_combine_kernel<bf16_t><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const bf16_t *)shared, shared_gate, n, d, top);
-        else moe_combine_kernel<float><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const float *)shared, shared_gate, n, d, top);
+        if (type == LCU_BF16) moe_combine_kernel<bf16_t><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const bf16_t *)shared, shared_gate, n, d, top, fresh);
+        else moe_combine_kernel<float><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const float *)shared, shared_gate, n, d, top, fresh);
         LCU_LAUNCH_CHECK();
     }
     return LCU_OK;

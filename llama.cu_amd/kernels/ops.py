@@ -1206,12 +1206,13 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, bias: Optional[to
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
                 out: torch.Tensor, gated: bool = False, shared: Optional[torch.Tensor] = None,
-                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                shared_gate: Optional[torch.Tensor] = None, fresh: bool = False) -> torch.Tensor:
     """``out[t] += sum over t's experts e of  w_down[e] @ gelu(w_up[e] @ (weight * h[t]))`` (the exact gelu; the
     weight scales what goes INTO the expert, not what comes out).  ``w_up [experts, ff, d]``, ``w_down [experts, d, ff]`` in ``h``'s type,
     ``out`` float32 ``[n, d]``.  ``gated``: ``out[t] += sum_e weight * w_down[e] @ (silu(gate[e] @ h[t]) * (up[e] @ h[t]))``
     with ``w_up [experts, 2 * ff, d]`` holding in turns 16 rows of the gate matrix and the 16 up rows that meet them
-    (``gated_rows`` lays them out so); ``shared [n, d]`` (with ``shared_gate [n]`` float32, or ones) is added beside."""
+    (``gated_rows`` lays them out so); ``shared [n, d]`` (with ``shared_gate [n]`` float32, or ones) is added beside;
+    ``fresh``: ``out`` is written, not added to (it need not hold anything)."""
     _gpu(h, ids, wts, w_up, w_down, out, shared, shared_gate)
     _rows(h, "moe input")
     for t, what in ((h, "moe input"), (ids, "moe ids"), (wts, "moe weights"), (w_up, "moe up"), (w_down, "moe down"), (out, "moe out")):
@@ -1229,6 +1230,8 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: tor
     per = 8 if h.dtype == torch.bfloat16 else 4
     if d % per or ff % (16 if gated else per):
         raise KernelError(f"moe_experts: the width {d} and the experts' {ff} must be multiples of {per} ({16 if gated else per} for the experts')")
+    if fresh and not gated:
+        raise KernelError("moe_experts: only the gated form writes its output afresh")
     if shared is not None:
         _contig(shared, "shared expert rows")
         if not gated or shared.shape != (n, d) or shared.dtype != h.dtype:
@@ -1244,7 +1247,8 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: tor
     y = torch.empty((total, d), dtype=torch.float32, device=h.device) if (top > 1 or gated) else None
     _check(lib.lcu_moe_experts(_ptr(h), _type(h, "moe input"), _ptr(ids), _ptr(wts), _ptr(ints), max_tiles, _ptr(w_up),
                                _ptr(w_down), _ptr(act), _ptr(y), _ptr(out), n, d, ff, experts, top, int(bool(gated)),
-                               _ptr(shared), _ptr(shared_gate if shared is not None else None), _stream()), "moe_experts")
+                               _ptr(shared), _ptr(shared_gate if shared is not None else None), int(bool(fresh)), _stream()),
+           "moe_experts")
     return out
 
 

@@ -149,11 +149,12 @@ class GatedMoE(Part):
     def forward(self, h):
         routed = ops.moe_route(h, self.router, self.top, bias=self.bias, softmax_chosen=True, extra=1 if self.shared is not None else 0)
         ids, wts = routed[0], routed[1]
-        out = torch.zeros((h.shape[0], self.hidden_size), dtype=torch.float32, device=h.device)
+        out = torch.empty((h.shape[0], self.hidden_size), dtype=torch.float32, device=h.device)
         if self.shared is not None:
-            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True, shared=self.shared.forward(h), shared_gate=routed[2])
+            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True, shared=self.shared.forward(h),
+                            shared_gate=routed[2], fresh=True)
         else:
-            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True)
+            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True, fresh=True)
         return out
 
 
