@@ -405,7 +405,7 @@ def ralepel_config(z, positions):
             kind, m = "attention", {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024}}
         else:
             kind, m = "latent_attention", {"heads": h, "dim": 96, "rot_dim": 32, "vdim": d, "kv_rank": 96, "scale": d ** -0.5,
-                                           "rot": {"dims": 32, "base": 50000.0}}
+                                           "rot": {"dims": 32, "base": 10000.0}}
             if i % 4 == 3 and last_latent is not None:
                 m["kv_from"] = last_latent
             else:
