@@ -513,11 +513,11 @@ def test_a_toy_position_encoding_that_is_a_bias_inside_the_scores():
         def score_slopes(self):
             return self.slopes
 
-    register_part("position", "distance_bias", DistanceBias, replace=True)
+    register_part("position", "toy_distance_bias", DistanceBias, replace=True)      # (a kind of its own: the package has one named distance_bias)
     cfg_d = dict(common.TINY_A)
     cfg = LlamaConfig.from_dict(cfg_d)
     spec = llama_spec(cfg)
-    spec.layers[0].params["mixer"].params["position"] = PartSpec("distance_bias", {"heads": cfg.num_attention_heads})
+    spec.layers[0].params["mixer"].params["position"] = PartSpec("toy_distance_bias", {"heads": cfg.num_attention_heads})
     runner, w = runner_for(spec, 17, "float32", max_tokens=512, max_seqs=3)
     nh, nkv, dh = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
 
