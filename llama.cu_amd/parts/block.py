@@ -225,33 +225,14 @@ class ParallelBlock(Part):
 register_part("block", "parallel", ParallelBlock)
 
 
-class SandwichBlock(Part):
-    """A norm in front of and behind every sublayer: ``x += post1(mixer(norm1(x)))``, then ``x += post2(ffn(norm2(x)))``.
-    The feed-forward (with its two norms) may be missing.  The four norms are RMS norms (a factor per row times a
-    weight per column).  The norm behind a sublayer, the residual sum and the norm in front of the next sublayer are
-    one kernel (``ops.norm_post``), also across the border to the next block where that block takes such rows
-    (``NormedRows``); the stream and the sums are 32-bit."""
-
-    def __init__(self, norm1: PartSpec, mixer: PartSpec, post1: PartSpec, norm2: Optional[PartSpec] = None,
-                 ffn: Optional[PartSpec] = None, post2: Optional[PartSpec] = None):
-        if len({norm2 is None, ffn is None, post2 is None}) != 1:
-            raise ValueError("sandwich block: the feed-forward and its two norms come together or not at all")
-        self.specs = {"norm1": norm1, "mixer": mixer, "post1": post1, "norm2": norm2, "ffn": ffn, "post2": post2}
-        self.norm1 = make_part("norm", norm1)
-        self.mixer = make_part("mixer", mixer)
-        self.post1 = make_part("norm", post1)
-        self.norm2 = make_part("norm", norm2) if norm2 is not None else None
-        self.ffn = make_part("ffn", ffn) if ffn is not None else None
-        self.post2 = make_part("norm", post2) if post2 is not None else None
-        for name in ("norm1", "post1", "norm2", "post2"):
-            part = getattr(self, name)
-            if part is not None and not part.deferrable:
-                raise ValueError(f"sandwich block: {name} must be a norm that is a factor per row times a weight per column")
-        self.graph_safe = all(p.graph_safe for _, p in self._children())
+class _SublayersInTurn(Part):
+    """What blocks that run a mixer and then a feed-forward share: their children's tensors under the children's names,
+    loading, fused groups, the mixer's cache need, ``prepare`` and the decode kernel's split.  A subclass keeps its
+    children's specifications in ``self.specs`` and names them, in order, in ``CHILDREN``."""
+    CHILDREN: tuple = ()
 
     def _children(self):
-        return [(self.specs[k].name, getattr(self, k)) for k in ("norm1", "mixer", "post1", "norm2", "ffn", "post2")
-                if getattr(self, k) is not None]
+        return [(self.specs[k].name, getattr(self, k)) for k in self.CHILDREN if getattr(self, k) is not None]
 
     def tensors(self) -> Dict[str, TensorSpec]:
         out = {}
@@ -281,6 +262,33 @@ class SandwichBlock(Part):
 
     def decode_splits(self, batch: int, max_ctx_len: int) -> int:
         return int(self.mixer.decode_splits(batch, max_ctx_len))
+
+
+class SandwichBlock(_SublayersInTurn):
+    """A norm in front of and behind every sublayer: ``x += post1(mixer(norm1(x)))``, then ``x += post2(ffn(norm2(x)))``.
+    The feed-forward (with its two norms) may be missing.  The four norms are RMS norms (a factor per row times a
+    weight per column).  The norm behind a sublayer, the residual sum and the norm in front of the next sublayer are
+    one kernel (``ops.norm_post``), also across the border to the next block where that block takes such rows
+    (``NormedRows``); the stream and the sums are 32-bit."""
+
+    CHILDREN = ("norm1", "mixer", "post1", "norm2", "ffn", "post2")
+
+    def __init__(self, norm1: PartSpec, mixer: PartSpec, post1: PartSpec, norm2: Optional[PartSpec] = None,
+                 ffn: Optional[PartSpec] = None, post2: Optional[PartSpec] = None):
+        if len({norm2 is None, ffn is None, post2 is None}) != 1:
+            raise ValueError("sandwich block: the feed-forward and its two norms come together or not at all")
+        self.specs = {"norm1": norm1, "mixer": mixer, "post1": post1, "norm2": norm2, "ffn": ffn, "post2": post2}
+        self.norm1 = make_part("norm", norm1)
+        self.mixer = make_part("mixer", mixer)
+        self.post1 = make_part("norm", post1)
+        self.norm2 = make_part("norm", norm2) if norm2 is not None else None
+        self.ffn = make_part("ffn", ffn) if ffn is not None else None
+        self.post2 = make_part("norm", post2) if post2 is not None else None
+        for name in ("norm1", "post1", "norm2", "post2"):
+            part = getattr(self, name)
+            if part is not None and not part.deferrable:
+                raise ValueError(f"sandwich block: {name} must be a norm that is a factor per row times a weight per column")
+        self.graph_safe = all(p.graph_safe for _, p in self._children())
 
     @property
     def first_norm(self):
@@ -312,13 +320,15 @@ class SandwichBlock(Part):
 register_part("block", "sandwich", SandwichBlock)
 
 
-class PostNormBlock(Part):
+class PostNormBlock(_SublayersInTurn):
     """A norm behind every sublayer and none in front: ``x += post1(mixer(x))``, then ``x += post2(ffn(x))``; the sublayers
     read the residual stream itself (rounded to the compute type).  The feed-forward, with its norm, may be missing.  The
     norms are RMS norms (a factor per row times a weight per column).  The norm behind a sublayer, the residual sum and
     the rounded copy of the new stream that the next sublayer reads are one kernel (``ops.norm_post``), also across the
     border to the next block where that block takes such rows; a bias that the mixer's last product still lacks is
     added in the same kernel.  The stream and the sums are 32-bit."""
+
+    CHILDREN = ("mixer", "post1", "ffn", "post2")
 
     def __init__(self, mixer: PartSpec, post1: PartSpec, ffn: Optional[PartSpec] = None, post2: Optional[PartSpec] = None):
         if (ffn is None) != (post2 is None):
@@ -335,17 +345,8 @@ class PostNormBlock(Part):
         self._reads = make_part("norm", PartSpec("none"))          # what stands where a first norm would
         self.graph_safe = all(p.graph_safe for _, p in self._children())
 
-    tensors = SandwichBlock.tensors
-    fused_groups = SandwichBlock.fused_groups
-    cache_need = SandwichBlock.cache_need
-    prepare = SandwichBlock.prepare
-    decode_splits = SandwichBlock.decode_splits
-
-    def _children(self):
-        return [(self.specs[k].name, getattr(self, k)) for k in ("mixer", "post1", "ffn", "post2") if getattr(self, k) is not None]
-
     def load(self, tensors, build: BuildContext) -> None:
-        SandwichBlock.load(self, tensors, build)
+        super().load(tensors, build)
         self._reads.load({}, build)
 
     @property
