@@ -87,7 +87,15 @@ CFG_E = config(64, 48, [
     {"type": "attention", "mixer": attention(6, 2, 8, 0.4, 40), "mlp": moe(4, 2, 16, shared=16)},
 ], eps=1e-5)
 
-CONFIGS = {"A": CFG_A, "B": CFG_B, "C": CFG_C, "D": CFG_D, "E": CFG_E}
+# groups of twenty heads on one key/value head, and twenty latent heads: more than the matrix-core kernels take in a
+# group, so that in bfloat16 these layers run on the generic kernel, with keys and values stored at those kernels' sizes
+CFG_F = config(80, 64, [
+    {"type": "latent_attention", "mixer": latent(20, 8, 8, 8, 48, 0.3, base=400.0), "mlp": dense(48)},
+    {"type": "attention", "mixer": attention(20, 1, 16, 0.35, 21), "mlp": moe(3, 2, 32, shared=16)},
+    {"type": "latent_attention", "mixer": latent(2, 24, 8, 16, 48, 0.3, base=400.0, kv_from=0), "mlp": None},
+], eps=1e-5)
+
+CONFIGS = {"A": CFG_A, "B": CFG_B, "C": CFG_C, "D": CFG_D, "E": CFG_E, "F": CFG_F}
 
 
 def sharpened(cfg: dict, factor: float) -> dict:

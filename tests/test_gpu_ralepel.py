@@ -312,12 +312,12 @@ def runner_for(folder, dtype, **kw):
 
 
 @pytest.mark.parametrize("name,dtype", [("A", "float32"), ("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"), ("C", "float32"),
-                                        ("C", "bfloat16"), ("D", "float32"), ("E", "float32")])
+                                        ("C", "bfloat16"), ("D", "float32"), ("E", "float32"), ("F", "float32"), ("F", "bfloat16")])
 def test_a_whole_prompt_against_the_plain_model(name, dtype):
     cfg, w, folder = model(name, dtype=dtype)
     toks = tokens_of(cfg["vocab"], 100, 1)
     want = plain_logits(cfg, w, toks)
-    r = runner_for(folder, dtype, page_size={"A": 16, "B": 32, "C": 48, "D": 64, "E": 16}[name])
+    r = runner_for(folder, dtype, page_size={"A": 16, "B": 32, "C": 48, "D": 64, "E": 16, "F": 16}[name])
     got = r.step([0], [toks], [list(range(len(toks)))])
     assert_close(got, want, REL[dtype], f"model {name} in {dtype}")
     r.end(0)
@@ -348,7 +348,7 @@ def test_models_of_one_kind_of_mixer_and_the_first_tokens_of_a_sequence(name, dt
     r.cache.check()
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "float32")])
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "float32"), ("F", "bfloat16")])
 def test_prefill_against_token_by_token_decoding_and_portions_down_to_two_tokens(name, dtype):
     cfg, w, folder = model(name, dtype=dtype)
     toks = tokens_of(cfg["vocab"], 90, 2)
