@@ -145,3 +145,23 @@ def test_routing_weights_add_up_to_one_over_the_chosen():
     assert ids.shape == (20, 2) and np.allclose(wts.sum(1), 1.0) and (wts[:, 0] >= wts[:, 1]).all()
     one = P.route(x, cfg["layers"][4]["mlp"], w, "l4.mlp.")[1]
     assert (one == 1.0).all()
+
+
+def test_the_bench_configurations_of_the_design_build_and_hold_the_dense_models_active_weights():
+    """``bench.py --workload designs``: the design's configuration at both sizes reads as a model, every second latent layer
+    reads the latent before it, and a mixture layer's active feed-forward weights are within a tenth of the dense model's."""
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for z in bench.DESIGN_SIZES.values():
+        cfg = bench.ralepel_config(z, 4096)
+        model = DecoderModel(architecture_of(cfg.to_dict()).build_spec(cfg))
+        assert len(model.layers) == z["layers"] and model.tensors()
+        assert any(e.cache_of is not None for e in model.spec.run_order)
+        dense = [l.ff for l in cfg.layers if isinstance(l.ff, int)][0]
+        for layer in cfg.layers:
+            if not isinstance(layer.ff, int):
+                active = layer.ff.top * layer.ff.expert_ff + layer.ff.shared_ff
+                assert abs(active - dense) <= 0.1 * dense
