@@ -5,9 +5,10 @@ from .llama import LlamaConfig
 from .divasun import DivasunConfig
 from .lozezen import LozezenConfig
 from .ralepel import RalepelConfig
+from .mufotar import MufotarConfig
 from .registry import (Architecture, architecture_of, register_architecture, registered_architectures, load_config,
                        load_plugins, load_plugins_from_env, PLUGINS_ENV)
 
-__all__ = ["ConfigError", "read_config_json", "LlamaConfig", "DivasunConfig", "LozezenConfig", "RalepelConfig", "Architecture", "architecture_of",
+__all__ = ["ConfigError", "read_config_json", "LlamaConfig", "DivasunConfig", "LozezenConfig", "RalepelConfig", "MufotarConfig", "Architecture", "architecture_of",
            "register_architecture", "registered_architectures", "load_config", "load_plugins", "load_plugins_from_env",
            "PLUGINS_ENV"]

@@ -87,8 +87,8 @@ constexpr int scan_groups() { return DK > 0 && DK % 32 == 0 ? 8 : 4; }
 
 template <class T, int DK>
 __global__ void __launch_bounds__(64)
-delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const float *__restrict__ prep,
-                  float *__restrict__ state, float *__restrict__ o, const int *__restrict__ q_start,
+delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const float *__restrict__ vf, const float *__restrict__ prep,
+                  float *__restrict__ state, size_t slot_stride, float *__restrict__ o, const int *__restrict__ q_start,
                   const int *__restrict__ ctx_len, const int *__restrict__ state_slot, int heads, int dk_rt, int dv) {
     const int r = blockIdx.x, h = blockIdx.y;
     const int t0 = q_start[r], t1 = q_start[r + 1];
@@ -101,7 +101,7 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
         const int g = threadIdx.x / SCAN_COLS, j = blockIdx.z * SCAN_COLS + threadIdx.x % SCAN_COLS;
         const bool live = j < dv;
         const int jj = live ? j : dv - 1;                     // lanes beyond dv compute along and store nothing
-        float *col = state + (((size_t)state_slot[r] * heads + h) * DK + g * SL) * dv + jj;   // S[g * SL + i][j] at col[i * dv]
+        float *col = state + (size_t)state_slot[r] * slot_stride + ((size_t)h * DK + g * SL) * dv + jj;   // S[g * SL + i][j] at col[i * dv]
         // a vector in LDS: the four groups' quarters, each followed by four floats of padding, so that the groups' reads of
         // their quarters (the same offset in each) fall into different banks
         constexpr int SLP = SL + 4, VEC = SCAN_GROUPS * SLP;
@@ -113,6 +113,7 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
         // token's own arithmetic is far shorter than a trip to memory
         float next[TB][PER_LANE], v_next[TB];
         const T *vp = proj + off_v + h * dv + jj;
+        const float *vfp = vf ? vf + h * dv + jj : nullptr;         // the values as 32-bit rows [n, heads * dv] of their own
         auto fetch = [&](int t) {
 #pragma unroll
             for (int b = 0; b < TB; ++b) {
@@ -123,7 +124,7 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
                     const int idx = e * 64 + threadIdx.x;
                     next[b][e] = idx < 5 * DK ? p[idx] : 0.f;
                 }
-                v_next[b] = to_f32(vp[(size_t)(t + b) * row_stride]);
+                v_next[b] = vfp ? vfp[(size_t)(t + b) * heads * dv] : to_f32(vp[(size_t)(t + b) * row_stride]);
             }
         };
         if (t0 < t1) fetch(t0);
@@ -170,11 +171,11 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
         const int dk = dk_rt, j = blockIdx.z * 64 + threadIdx.x;
         const bool live = j < dv;
         const int jj = live ? j : dv - 1;
-        float *col = state + (((size_t)state_slot[r] * heads + h) * dk) * dv + jj;     // S[i][j] at col[i * dv]
+        float *col = state + (size_t)state_slot[r] * slot_stride + ((size_t)h * dk) * dv + jj;     // S[i][j] at col[i * dv]
         if (fresh && live)
             for (int i = 0; i < dk; ++i) col[(size_t)i * dv] = 0.f;
         for (int t = t0; t < t1; ++t) {
-            const float v = to_f32(proj[(size_t)t * row_stride + off_v + h * dv + jj]);
+            const float v = vf ? vf[(size_t)t * heads * dv + h * dv + jj] : to_f32(proj[(size_t)t * row_stride + off_v + h * dv + jj]);
             const float *p = prep + ((size_t)t * heads + h) * 5 * dk;
             float us = 0.f, acc = 0.f;
             for (int i = 0; i < dk; ++i) us += p[2 * dk + i] * col[(size_t)i * dv];
@@ -205,16 +206,12 @@ delta_out_kernel(const float *__restrict__ o, const T *__restrict__ proj, int ro
     }
 }
 
+// The scan over the step's tokens for every head size it is compiled for.  vf: null, or the values as 32-bit rows.
 template <class T>
-static int delta_rule_t(const T *proj, int row_stride, int off_r, int off_k, int off_v, int off_g, int off_a, int off_l,
-                        const float *w2, const float *w0, const float *a_bias, const float *weight, float *prep,
-                        float *o, float *state, T *out, const int *q_start, const int *ctx_len, const int *state_slot,
-                        int n, int n_req, int heads, int dk, int dv, int rank, float eps, hipStream_t stream) {
-    int threads = ((dk > rank ? dk : rank) + 63) / 64 * 64;
-    if (threads > 256) threads = 256;
-    delta_prep_kernel<T><<<dim3(n, heads), dim3(threads), 0, stream>>>(proj, row_stride, off_r, off_k, off_a, off_l, w2, w0, a_bias, prep, heads, dk, rank);
-    LCU_LAUNCH_CHECK();
-#define SCAN(DK) delta_scan_kernel<T, DK><<<dim3(n_req, heads, (dv + (DK ? 64 / scan_groups<T, DK>() : 64) - 1) / (DK ? 64 / scan_groups<T, DK>() : 64)), dim3(64), 0, stream>>>(proj, row_stride, off_v, prep, state, o, q_start, ctx_len, state_slot, heads, dk, dv)
+static int delta_scan_launch(const T *proj, int row_stride, int off_v, const float *vf, const float *prep, float *state,
+                             size_t slot_stride, float *o, const int *q_start, const int *ctx_len, const int *state_slot,
+                             int n_req, int heads, int dk, int dv, hipStream_t stream) {
+#define SCAN(DK) delta_scan_kernel<T, DK><<<dim3(n_req, heads, (dv + (DK ? 64 / scan_groups<T, DK>() : 64) - 1) / (DK ? 64 / scan_groups<T, DK>() : 64)), dim3(64), 0, stream>>>(proj, row_stride, off_v, vf, prep, state, slot_stride, o, q_start, ctx_len, state_slot, heads, dk, dv)
     switch (dk) {
     case 16: SCAN(16); break;
     case 32: SCAN(32); break;
@@ -230,6 +227,21 @@ static int delta_rule_t(const T *proj, int row_stride, int off_r, int off_k, int
     }
 #undef SCAN
     LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+template <class T>
+static int delta_rule_t(const T *proj, int row_stride, int off_r, int off_k, int off_v, int off_g, int off_a, int off_l,
+                        const float *w2, const float *w0, const float *a_bias, const float *weight, float *prep,
+                        float *o, float *state, T *out, const int *q_start, const int *ctx_len, const int *state_slot,
+                        int n, int n_req, int heads, int dk, int dv, int rank, float eps, hipStream_t stream) {
+    int threads = ((dk > rank ? dk : rank) + 63) / 64 * 64;
+    if (threads > 256) threads = 256;
+    delta_prep_kernel<T><<<dim3(n, heads), dim3(threads), 0, stream>>>(proj, row_stride, off_r, off_k, off_a, off_l, w2, w0, a_bias, prep, heads, dk, rank);
+    LCU_LAUNCH_CHECK();
+    const int rc = delta_scan_launch<T>(proj, row_stride, off_v, nullptr, prep, state, (size_t)heads * dk * dv, o, q_start, ctx_len,
+                                        state_slot, n_req, heads, dk, dv, stream);
+    if (rc != LCU_OK) return rc;
     delta_out_kernel<T><<<dim3(n, heads), dim3(64), 0, stream>>>(o, proj, row_stride, off_g, weight, out, heads, dv, eps);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
@@ -250,4 +262,90 @@ LCU_API int lcu_delta_rule(const void *proj, int type, int row_stride, int off_r
     if (type == LCU_BF16)
         return delta_rule_t<bf16_t>((const bf16_t *)proj, row_stride, off_r, off_k, off_v, off_g, off_a, off_l, w2, w0, a_bias, weight, prep, o, state, (bf16_t *)out, q_start, ctx_len, state_slot, n, n_req, heads, dk, dv, rank, eps, stream);
     return LCU_BAD_ARGUMENT;
+}
+
+// ---------------------------------------------------------------- the gated delta rule
+// One decay and one rate per head and token:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q,  with q and k
+// unit vectors per head (q also times dk^-1/2).  Written out, S <- g S - (beta g k)(k^T S) + k (beta v)^T with S as the
+// token found it: the scan above with the decay g on every key channel, the removal vector beta g k, and the values
+// beta v.  Several value heads may share one query/key head (`group` of them).
+//   prep (parallel over tokens and value heads): the scan's five vectors and the values times beta;
+//   out  (parallel): o of each head divided by its root mean square, times a weight, times silu(gate).
+// qkv: [n, qk_heads * dk (q) | qk_heads * dk (k) | heads * dv (v)] 32-bit, the projections behind their convolutions
+// and activations.  rows: [n, row_stride] 32-bit holding per head the decay's and the rate's projections at columns
+// off_a and off_b, and the gate's heads * dv columns at off_g.
+__device__ __forceinline__ float softplus_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+__global__ void gated_delta_prep_kernel(const float *__restrict__ qkv, const float *__restrict__ rows, int row_stride, int off_a,
+                                        int off_b, const float *__restrict__ a_log, const float *__restrict__ dt_bias,
+                                        float *__restrict__ prep, float *__restrict__ vb, int heads, int group, int dk, int dv) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, h = blockIdx.y, qh = h / group, qk_heads = heads / group;
+    const int width = 2 * qk_heads * dk + heads * dv;
+    const float *q = qkv + (size_t)t * width + qh * dk, *k = q + qk_heads * dk;
+    const float *v = qkv + (size_t)t * width + 2 * qk_heads * dk + h * dv;
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+        sq += q[i] * q[i];
+        sk += k[i] * k[i];
+    }
+    sq = block_sum(sq, scratch);
+    sk = block_sum(sk, scratch);
+    const float qf = 1.0f / sqrtf(sq + 1e-6f) / sqrtf((float)dk), kf = 1.0f / sqrtf(sk + 1e-6f);
+    const float *row = rows + (size_t)t * row_stride;
+    const float beta = sigmoidf_(row[off_b + h]);
+    const float g = expf(-expf(a_log[h]) * softplus_(row[off_a + h] + dt_bias[h]));
+    float *out = prep + ((size_t)t * heads + h) * 5 * dk;
+    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+        const float u = k[i] * kf;
+        out[i] = g;
+        out[dk + i] = beta * g * u;
+        out[2 * dk + i] = u;
+        out[3 * dk + i] = u;
+        out[4 * dk + i] = q[i] * qf;
+    }
+    for (int j = threadIdx.x; j < dv; j += blockDim.x) vb[((size_t)t * heads + h) * dv + j] = beta * v[j];
+}
+
+// One wave per (token, head): out = o / rms(o) * weight * silu(gate); weight: [dv], shared by the heads.
+template <class T>
+__global__ void __launch_bounds__(64)
+gated_delta_out_kernel(const float *__restrict__ o, const float *__restrict__ rows, int row_stride, int off_g,
+                       const float *__restrict__ weight, T *__restrict__ out, int heads, int dv, float eps) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const float *oh = o + (size_t)t * heads * dv + h * dv;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < dv; j += 64) ss += oh[j] * oh[j];
+    const float f = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+    for (int j = threadIdx.x; j < dv; j += 64) {
+        const float z = rows[(size_t)t * row_stride + off_g + h * dv + j];
+        out[(size_t)t * heads * dv + h * dv + j] = from_f32<T>(oh[j] * f * weight[j] * (z / (1.0f + expf(-z))));
+    }
+}
+
+// a_log, dt_bias: [heads]; weight: [dv], 32-bit.  prep: scratch [n, heads, 5, dk]; vb, o: scratch [n, heads * dv], 32-bit.
+// state: slot s at state + s * slot_stride, [heads, dk, dv] 32-bit.  out: [n, heads * dv] of out_type.
+LCU_API int lcu_gated_delta_rule(const float *qkv, const float *rows, int row_stride, int off_a, int off_b, int off_g,
+                                 const float *a_log, const float *dt_bias, const float *weight, float *prep, float *vb, float *o,
+                                 float *state, long long slot_stride, void *out, int out_type, const int *q_start,
+                                 const int *ctx_len, const int *state_slot, int n, int n_req, int heads, int qk_heads, int dk,
+                                 int dv, float eps, hipStream_t stream) {
+    if (n <= 0 || n_req <= 0) return LCU_OK;
+    if (heads <= 0 || heads > 65535 || qk_heads <= 0 || heads % qk_heads || dk <= 0 || dv <= 0 || dv > 8 * 65535 ||
+        (out_type != LCU_F32 && out_type != LCU_BF16))
+        return LCU_BAD_ARGUMENT;
+    int threads = ((dk > dv ? dk : dv) + 63) / 64 * 64;
+    if (threads > 256) threads = 256;
+    gated_delta_prep_kernel<<<dim3(n, heads), dim3(threads), 0, stream>>>(qkv, rows, row_stride, off_a, off_b, a_log, dt_bias, prep, vb,
+                                                                           heads, heads / qk_heads, dk, dv);
+    LCU_LAUNCH_CHECK();
+    const int rc = delta_scan_launch<float>(nullptr, 0, 0, vb, prep, state, (size_t)slot_stride, o, q_start, ctx_len, state_slot, n_req,
+                                            heads, dk, dv, stream);
+    if (rc != LCU_OK) return rc;
+    if (out_type == LCU_F32)
+        gated_delta_out_kernel<float><<<dim3(n, heads), dim3(64), 0, stream>>>(o, rows, row_stride, off_g, weight, (float *)out, heads, dv, eps);
+    else
+        gated_delta_out_kernel<bf16_t><<<dim3(n, heads), dim3(64), 0, stream>>>(o, rows, row_stride, off_g, weight, (bf16_t *)out, heads, dv, eps);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
 }

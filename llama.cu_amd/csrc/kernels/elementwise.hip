@@ -255,23 +255,30 @@ LCU_API int lcu_residual_add(float *x, const void *delta, int delta_type, long l
 }
 
 // ---------------------------------------------------------------- SwiGLU
-// out[r, c] = gate * (1 / (1 + exp(-gate))) * up with gate = gu[r, c], up = gu[r, di + c].
-template <class T>
+// out[r, c] = act(gate) * up with gate = gu[r, c], up = gu[r, di + c];  ACT 0: gate * (1 / (1 + exp(-gate))) (silu),
+// 1: the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
+enum { GATE_SILU = 0, GATE_GELU_TANH = 1 };
+template <int ACT>
+__device__ __forceinline__ float gate_act(float z) {
+    if (ACT == GATE_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z * (1.0f / (1.0f + expf(-z)));
+}
+
+template <class T, int ACT>
 __global__ void swiglu_kernel(T *__restrict__ out, const T *__restrict__ gu, int di) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= di) return;
     const size_t r = blockIdx.y;
     const float gate = to_f32(gu[r * 2 * di + c]);
     const float up = to_f32(gu[r * 2 * di + di + c]);
-    const float sig = 1.0f / (1.0f + expf(-gate));
-    out[r * di + c] = from_f32<T>(gate * sig * up);
+    out[r * di + c] = from_f32<T>(gate_act<ACT>(gate) * up);
 }
 
 // The same, eight neighbouring columns per thread (16-byte loads of bfloat16, 32-byte of
 // float32); for widths that are multiples of 8.
 template <class T> struct alignas(8 * sizeof(T)) Vec8 { T v[8]; };
 
-template <class T>
+template <class T, int ACT>
 __global__ void swiglu_vec8_kernel(T *__restrict__ out, const T *__restrict__ gu, int di) {
     const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
     if (c >= di) return;
@@ -282,36 +289,54 @@ __global__ void swiglu_vec8_kernel(T *__restrict__ out, const T *__restrict__ gu
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const float gate = to_f32(g.v[e]);
-        o.v[e] = from_f32<T>(gate * (1.0f / (1.0f + expf(-gate))) * to_f32(u.v[e]));
+        o.v[e] = from_f32<T>(gate_act<ACT>(gate) * to_f32(u.v[e]));
     }
     *(Vec8<T> *)(out + r * di + c) = o;
 }
 
-LCU_API int lcu_swiglu(void *out, const void *gate_up, int type, int n, int di, hipStream_t stream) {
+template <class T, int ACT>
+static void swiglu_launch(T *out, const T *gate_up, int rows, int di, hipStream_t stream) {
+    const dim3 block(256);
+    if (di % 8 == 0)
+        swiglu_vec8_kernel<T, ACT><<<dim3((di / 8 + 255) / 256, rows), block, 0, stream>>>(out, gate_up, di);
+    else
+        swiglu_kernel<T, ACT><<<dim3((di + 255) / 256, rows), block, 0, stream>>>(out, gate_up, di);
+}
+
+// act: 0 silu, 1 the tanh form of gelu.
+LCU_API int lcu_swiglu(void *out, const void *gate_up, int type, int n, int di, int act, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
-    if (di <= 0) return LCU_BAD_ARGUMENT;
-    dim3 block(256);
+    if (di <= 0 || (act != GATE_SILU && act != GATE_GELU_TANH) || (type != LCU_F32 && type != LCU_BF16)) return LCU_BAD_ARGUMENT;
     // grid.y is limited to 65535 rows: larger batches go in slices
     for (int r0 = 0; r0 < n; r0 += 65535) {
         const int rows = (n - r0) < 65535 ? (n - r0) : 65535;
-        dim3 grid((di + 255) / 256, rows);
-        if (di % 8 == 0) {
-            dim3 vgrid((di / 8 + 255) / 256, rows);
-            if (type == LCU_F32)
-                swiglu_vec8_kernel<float><<<vgrid, block, 0, stream>>>((float *)out + (size_t)r0 * di, (const float *)gate_up + (size_t)r0 * 2 * di, di);
-            else if (type == LCU_BF16)
-                swiglu_vec8_kernel<bf16_t><<<vgrid, block, 0, stream>>>((bf16_t *)out + (size_t)r0 * di, (const bf16_t *)gate_up + (size_t)r0 * 2 * di, di);
-            else
-                return LCU_BAD_ARGUMENT;
-            continue;
+        if (type == LCU_F32) {
+            float *o = (float *)out + (size_t)r0 * di;
+            const float *g = (const float *)gate_up + (size_t)r0 * 2 * di;
+            if (act == GATE_SILU) swiglu_launch<float, GATE_SILU>(o, g, rows, di, stream);
+            else swiglu_launch<float, GATE_GELU_TANH>(o, g, rows, di, stream);
+        } else {
+            bf16_t *o = (bf16_t *)out + (size_t)r0 * di;
+            const bf16_t *g = (const bf16_t *)gate_up + (size_t)r0 * 2 * di;
+            if (act == GATE_SILU) swiglu_launch<bf16_t, GATE_SILU>(o, g, rows, di, stream);
+            else swiglu_launch<bf16_t, GATE_GELU_TANH>(o, g, rows, di, stream);
         }
-        if (type == LCU_F32)
-            swiglu_kernel<float><<<grid, block, 0, stream>>>((float *)out + (size_t)r0 * di, (const float *)gate_up + (size_t)r0 * 2 * di, di);
-        else if (type == LCU_BF16)
-            swiglu_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t *)out + (size_t)r0 * di, (const bf16_t *)gate_up + (size_t)r0 * 2 * di, di);
-        else
-            return LCU_BAD_ARGUMENT;
     }
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// ---------------------------------------------------------------- a cap on the logits
+// x <- cap * tanh(x / cap), in place, 32-bit.
+__global__ void softcap_kernel(float *__restrict__ x, size_t total, float cap) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) x[i] = cap * tanhf(x[i] / cap);
+}
+
+LCU_API int lcu_softcap(float *x, long long total, float cap, hipStream_t stream) {
+    if (total <= 0) return LCU_OK;
+    if (!(cap > 0.f)) return LCU_BAD_ARGUMENT;
+    softcap_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream>>>(x, (size_t)total, cap);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }

@@ -2,8 +2,10 @@
 //
 //   route:   z = W_router h (+ bias) (32-bit), the `top` experts with the largest z (ties: the lower
 //            index), each with the weight sigmoid(z) (a token's weights are not made to add up to one) or,
-//            in the other mode, with the softmax over the chosen logits alone; rows of the router's matrix
-//            behind the experts' are gates: sigmoid of their logit goes out per token;
+//            in the other mode, with the softmax over the chosen logits alone; or, in a third, with scores s = softmax(z)
+//            over all experts, the choice by s + a correction per expert, and the chosen scores divided by their sum as
+//            weights; rows of the router's matrix behind the experts' are gates: sigmoid of their logit goes out per
+//            token; the last experts may be identity experts, which have no matrices and return their input;
 //   group:   the (token, choice) pairs sorted by expert and cut into tiles of up to 16 or 64 rows of
 //            one expert, on the device (nothing comes back to the host);
 //   up:      act = gelu(W_up[e] (weight * h))    the weight scales what goes INTO the expert; or, gated:
@@ -32,7 +34,8 @@ template <class T> struct alignas(8 * sizeof(T)) Row8 { T v[8]; };
 constexpr int ROUTE_CHUNKS = 8;                  // rows of up to 8 * 512 elements stay in registers
 
 // bias: null or [experts], added to the logits.  mode 0: the weight of a chosen expert is sigmoid(z); 1: the softmax over
-// the chosen logits.  extra: rows of `router` behind the experts' (at most MOE_MAX_EXTRA); gates [n, extra] takes sigmoid
+// the chosen logits; 2: s = softmax(z) over all experts, the choice goes by s + bias (the bias is not added to the
+// logits), the weights are the chosen s divided by their sum + 1e-20.  extra: rows of `router` behind the experts' (at most MOE_MAX_EXTRA); gates [n, extra] takes sigmoid
 // of their logits (they are no experts and are never chosen).
 constexpr int MOE_MAX_EXTRA = 8;
 template <class T, int THREADS>
@@ -41,6 +44,8 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, cons
                  float *__restrict__ wts, float *__restrict__ gates, int d, int n_experts, int top, int mode, int extra) {
     __shared__ float z[MOE_MAX_EXPERTS + MOE_MAX_EXTRA];
     __shared__ float zc[MOE_MAX_EXPERTS];
+    __shared__ float sc[MOE_MAX_EXPERTS];
+    const float *logit_bias = mode == 2 ? nullptr : bias;
     const int experts = n_experts + extra;          // rows of the router's matrix
     const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const T *row = h + (size_t)t * d;
@@ -70,7 +75,7 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, cons
                 }
             }
             acc = wave_sum(acc);
-            if (lane == 0) z[e] = acc + (bias && e < n_experts ? bias[e] : 0.f);
+            if (lane == 0) z[e] = acc + (logit_bias && e < n_experts ? logit_bias[e] : 0.f);
         }
     } else {
         for (int e = wave; e < experts; e += THREADS / WAVE) {
@@ -78,11 +83,27 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, cons
             float acc = 0.f;
             for (int c = lane; c < d; c += WAVE) acc += to_f32(row[c]) * w[c];
             acc = wave_sum(acc);
-            if (lane == 0) z[e] = acc + (bias && e < n_experts ? bias[e] : 0.f);
+            if (lane == 0) z[e] = acc + (logit_bias && e < n_experts ? logit_bias[e] : 0.f);
         }
     }
     __syncthreads();
     for (int e = threadIdx.x; e < extra; e += THREADS) gates[(size_t)t * extra + e] = 1.0f / (1.0f + expf(-z[n_experts + e]));
+    if (mode == 2) {                                 // scores over all experts; z becomes what the choice goes by
+        if (wave == 0) {
+            float m = -INFINITY;
+            for (int e = lane; e < n_experts; e += WAVE) m = fmaxf(m, z[e]);
+            m = wave_max(m);
+            float part = 0.f;
+            for (int e = lane; e < n_experts; e += WAVE) part += expf(z[e] - m);
+            const float sum = wave_sum(part);
+            for (int e = lane; e < n_experts; e += WAVE) {
+                const float s = expf(z[e] - m) / sum;
+                sc[e] = s;
+                z[e] = s + (bias ? bias[e] : 0.f);
+            }
+        }
+        __syncthreads();
+    }
     for (int k = 0; k < top; ++k) {                  // the first wave chooses; the others only keep the barriers
         if (wave == 0) {
             float best = -INFINITY;
@@ -100,12 +121,18 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, cons
             if (arg >= n_experts) arg = 0;               // every logit NaN: any expert
             if (lane == 0) {
                 ids[(size_t)t * top + k] = arg;
-                zc[k] = z[arg];
+                zc[k] = mode == 2 ? sc[arg] : z[arg];
                 if (mode == 0) wts[(size_t)t * top + k] = 1.0f / (1.0f + expf(-z[arg]));
                 z[arg] = -INFINITY;
             }
         }
         __syncthreads();
+    }
+    if (mode == 2 && wave == 0) {                    // the chosen scores, made to add up to one
+        float part = 0.f;
+        for (int k = lane; k < top; k += WAVE) part += zc[k];
+        const float sum = wave_sum(part) + 1e-20f;
+        for (int k = lane; k < top; k += WAVE) wts[(size_t)t * top + k] = zc[k] / sum;
     }
     if (mode == 1 && wave == 0) {                    // the softmax over the chosen logits (the first is the largest)
         const float z0 = zc[0];
@@ -119,11 +146,12 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, cons
 // ---------------------------------------------------------------- group
 // One block.  ids: [total] experts of the (token, choice) pairs in flat order.  Writes
 // sorted_to_flat [total] (the pairs sorted by expert), and the tiles of up to rows_per_tile rows:
-// tile_expert, tile_begin (first sorted row), tile_rows, each [max_tiles], and n_tiles [1].
+// tile_expert, tile_begin (first sorted row), tile_rows, each [max_tiles], and n_tiles [1].  Only the first `tiled`
+// experts get tiles: the ones behind them have no matrices (identity experts), and their pairs are only sorted.
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int *__restrict__ ids, int total, int experts, int *__restrict__ sorted_to_flat,
                  int *__restrict__ tile_expert, int *__restrict__ tile_begin, int *__restrict__ tile_rows,
-                 int *__restrict__ n_tiles, int max_tiles, int rows_per_tile) {
+                 int *__restrict__ n_tiles, int max_tiles, int rows_per_tile, int tiled) {
     __shared__ int count[MOE_MAX_EXPERTS];
     __shared__ int cursor[MOE_MAX_EXPERTS];
     for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
@@ -134,7 +162,7 @@ moe_group_kernel(const int *__restrict__ ids, int total, int experts, int *__res
         int at = 0, tiles = 0;
         for (int e = 0; e < experts; ++e) {
             cursor[e] = at;
-            for (int r = 0; r < count[e] && tiles < max_tiles; r += rows_per_tile) {
+            for (int r = 0; e < tiled && r < count[e] && tiles < max_tiles; r += rows_per_tile) {
                 tile_expert[tiles] = e;
                 tile_begin[tiles] = at + r;
                 tile_rows[tiles] = count[e] - r < rows_per_tile ? count[e] - r : rows_per_tile;
@@ -400,15 +428,21 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
 }
 
 // out[t, c] (+)= sum_k wts[t, k] * y[t * top + k, c]  (in the order of k; wts null: ones)  + gate[t] * shared[t, c]  (shared null: nothing)
-// fresh: out is written, not added to (what it held is not read).
+// fresh: out is written, not added to (what it held is not read).  ids (null: none), real, h: a pair whose expert is
+// `real` or beyond is an identity expert, whose output is the token's input row h[t] itself.
 template <class T>
 __global__ void moe_combine_kernel(float *__restrict__ out, const float *__restrict__ y, const float *__restrict__ wts,
-                                   const T *__restrict__ shared, const float *__restrict__ gate, int n, int d, int top, int fresh) {
+                                   const T *__restrict__ shared, const float *__restrict__ gate, int n, int d, int top, int fresh,
+                                   const int *__restrict__ ids, int real, const T *__restrict__ h) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= d) return;
     for (size_t t = blockIdx.y; t < (size_t)n; t += gridDim.y) {
         float acc = fresh ? 0.f : out[t * d + c];
-        for (int k = 0; k < top; ++k) acc += (wts ? wts[t * top + k] : 1.f) * y[(t * top + k) * d + c];
+        for (int k = 0; k < top; ++k) {
+            const float w = wts ? wts[t * top + k] : 1.f;
+            if (ids && ids[t * top + k] >= real) acc += w * to_f32(h[t * d + c]);
+            else acc += w * y[(t * top + k) * d + c];
+        }
         if (shared) acc += (gate ? gate[t] : 1.f) * to_f32(shared[t * d + c]);
         out[t * d + c] = acc;
     }
@@ -424,7 +458,7 @@ LCU_API int lcu_moe_tile_rows(int total, int experts) { return (long long)total 
 LCU_API int lcu_moe_route(const void *h, int type, const float *router, const float *bias, int *ids, float *wts, float *gates,
                           int n, int d, int experts, int top, int mode, int extra, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
-    if (d <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts || (mode != 0 && mode != 1) ||
+    if (d <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts || mode < 0 || mode > 2 ||
         extra < 0 || extra > MOE_MAX_EXTRA || (extra && !gates))
         return LCU_BAD_ARGUMENT;
     const bool few = n <= 256 && experts > 4;
@@ -443,21 +477,23 @@ LCU_API int lcu_moe_route(const void *h, int type, const float *router, const fl
 // [total, d] 32-bit (only read and written when top > 1 or gated).  out: [n, d] 32-bit, added to.
 // gated: w_up is [experts, 2 * ff, d], in turns 16 rows of the gate matrix and the 16 rows of the up matrix that meet
 // them (ff a multiple of 16); act = silu(gate h) * (up h), and the weight scales what comes out; fresh: out is written
-// and not added to.  shared (null or
+// and not added to.  identity: ids may name experts + identity experts; the last `identity` have no matrices and return the
+// token's input.  shared (null or
 // [n, d] of `type`) with shared_gate (null or [n] 32-bit): rows that are added beside the experts', times the gate.
 LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float *wts, int *ints, int max_tiles,
                             const void *w_up, const void *w_down, void *act, float *y, float *out, int n, int d, int ff,
                             int experts, int top, int gated, const void *shared, const float *shared_gate, int fresh,
-                            hipStream_t stream) {
+                            int identity, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     const int per = type == LCU_BF16 ? 8 : 4;
     if (d <= 0 || ff <= 0 || d % per || ff % per || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || max_tiles <= 0 ||
-        (type != LCU_F32 && type != LCU_BF16) || (gated && ff % 16) || (shared && !gated) || (fresh && !gated))
+        (type != LCU_F32 && type != LCU_BF16) || (gated && ff % 16) || (shared && !gated) || (fresh && !gated) || identity < 0 ||
+        (identity && !gated) || experts + identity > MOE_MAX_EXPERTS)
         return LCU_BAD_ARGUMENT;
     const int total = n * top;
     const int tile_rows = lcu_moe_tile_rows(total, experts);
     int *sorted = ints, *t_exp = ints + total, *t_beg = t_exp + max_tiles, *t_rows = t_beg + max_tiles, *n_tiles = t_rows + max_tiles;
-    moe_group_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, total, experts, sorted, t_exp, t_beg, t_rows, n_tiles, max_tiles, tile_rows);
+    moe_group_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, total, experts + identity, sorted, t_exp, t_beg, t_rows, n_tiles, max_tiles, tile_rows, experts);
     LCU_LAUNCH_CHECK();
     const int add = top == 1 && !gated;
     float *down_to = add ? out : y;
@@ -487,8 +523,9 @@ LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float
     LCU_LAUNCH_CHECK();
     if (!add) {
         const dim3 gc((d + 255) / 256, n < 65535 ? n : 65535);
-        if (type == LCU_BF16) moe_combine_kernel<bf16_t><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const bf16_t *)shared, shared_gate, n, d, top, fresh);
-        else moe_combine_kernel<float><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const float *)shared, shared_gate, n, d, top, fresh);
+        const int *idp = identity ? ids : nullptr;
+        if (type == LCU_BF16) moe_combine_kernel<bf16_t><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const bf16_t *)shared, shared_gate, n, d, top, fresh, idp, experts, (const bf16_t *)h);
+        else moe_combine_kernel<float><<<gc, dim3(256), 0, stream>>>(out, y, gated ? wts : nullptr, (const float *)shared, shared_gate, n, d, top, fresh, idp, experts, (const float *)h);
         LCU_LAUNCH_CHECK();
     }
     return LCU_OK;

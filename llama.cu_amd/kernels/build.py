@@ -37,7 +37,7 @@ HIP_FLAGS += os.environ.get("LCU_HIP_FLAGS", "").split()
 
 KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "attention_mfma_bias", "gemm_generic", "gemm_skinny",
                     "gemm_mid", "sampling", "random_fill", "norm_conv", "qk_norm", "delta_rule", "moe", "norm_post", "qkv_prepare",
-                    "retention", "rglru", "latent"]
+                    "retention", "rglru", "latent", "causal_conv", "selective_scan"]
 HOST_LIBRARY = "host"
 
 _loaded: Dict[str, ctypes.CDLL] = {}

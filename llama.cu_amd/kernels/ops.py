@@ -210,8 +210,14 @@ def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return x
 
 
-def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``out = gate * sigmoid(gate) * up`` for ``gate_up = [gate | up]`` of shape ``[n, 2*di]``."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None, activation: str = "silu") -> torch.Tensor:
+    """``out = act(gate) * up`` for ``gate_up = [gate | up]`` of shape ``[n, 2*di]``; ``activation``: ``silu`` (``gate *
+    sigmoid(gate)``) or ``gelu_tanh`` (``0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))``)."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"swiglu: no activation {activation!r}; known: {sorted(GATE_ACTIVATIONS)}")
     _gpu(gate_up, out)
     _rows(gate_up, "gate_up"); _contig(gate_up, "gate_up")
     n, two_di = gate_up.shape
@@ -223,8 +229,19 @@ def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.T
     if out.shape != (n, di) or out.dtype != gate_up.dtype or not out.is_contiguous():
         raise KernelError("swiglu out: wrong shape, type or layout")
     lib = build.load("elementwise")
-    _check(lib.lcu_swiglu(_ptr(out), _ptr(gate_up), _type(gate_up, "gate_up"), n, di, _stream()), "swiglu")
+    _check(lib.lcu_swiglu(_ptr(out), _ptr(gate_up), _type(gate_up, "gate_up"), n, di, GATE_ACTIVATIONS[activation], _stream()), "swiglu")
     return out
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place (``x`` float32)."""
+    _gpu(x)
+    _contig(x, "softcap x")
+    if x.dtype != torch.float32 or not cap > 0:
+        raise KernelError("softcap: x must be float32 and the cap positive")
+    lib = build.load("elementwise")
+    _check(lib.lcu_softcap(_ptr(x), ctypes.c_longlong(x.numel()), ctypes.c_float(cap), _stream()), "softcap")
+    return x
 
 
 def feed_tokens(tokens: torch.Tensor, sampled: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
@@ -1181,10 +1198,12 @@ def delta_rule(proj: torch.Tensor, offsets: Dict[str, int], w2_t: torch.Tensor, 
 
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, bias: Optional[torch.Tensor] = None, softmax_chosen: bool = False,
-              extra: int = 0):
+              extra: int = 0, softmax_all: bool = False):
     """``(ids, weights)``, each ``[n, top]``: every row's ``top`` experts by ``router @ h + bias`` (32-bit; ties go to the
     lower index), largest first, with the weight ``sigmoid`` of that logit or, with ``softmax_chosen``, the softmax over
-    the chosen logits alone.  ``extra``: the last ``extra`` rows of ``router`` are no experts but gates; then a third
+    the chosen logits alone; with ``softmax_all`` the scores are ``s = softmax(router @ h)`` over all experts, the choice goes
+    by ``s + bias`` (the bias is a correction of the choice and not of the logits) and the weights are the chosen ``s``
+    divided by their sum + 1e-20.  ``extra``: the last ``extra`` rows of ``router`` are no experts but gates; then a third
     result ``[n, extra]`` holds ``sigmoid`` of their logits."""
     _gpu(h, router, bias)
     _rows(h, "moe input"); _contig(h, "moe input"); _contig(router, "router")
@@ -1195,24 +1214,27 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, bias: Optional[to
     if not 0 < top <= experts or experts > 1024 or not 0 <= extra <= 8:
         raise KernelError(f"moe_route: top {top} of {experts} experts is not supported (at most 1024 experts, 8 gates)")
     _f32_vec(bias, "router bias", experts)
+    if softmax_all and softmax_chosen:
+        raise KernelError("moe_route: the softmax runs over all experts or over the chosen ones, not both")
     ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
     wts = torch.empty((n, top), dtype=torch.float32, device=h.device)
     gates = torch.empty((n, extra), dtype=torch.float32, device=h.device) if extra else None
     lib = build.load("moe")
     _check(lib.lcu_moe_route(_ptr(h), _type(h, "moe input"), _ptr(router), _ptr(bias), _ptr(ids), _ptr(wts), _ptr(gates), n, d,
-                             experts, top, int(bool(softmax_chosen)), int(extra), _stream()), "moe_route")
+                             experts, top, 2 if softmax_all else int(bool(softmax_chosen)), int(extra), _stream()), "moe_route")
     return (ids, wts, gates) if extra else (ids, wts)
 
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
                 out: torch.Tensor, gated: bool = False, shared: Optional[torch.Tensor] = None,
-                shared_gate: Optional[torch.Tensor] = None, fresh: bool = False) -> torch.Tensor:
+                shared_gate: Optional[torch.Tensor] = None, fresh: bool = False, identity: int = 0) -> torch.Tensor:
     """``out[t] += sum over t's experts e of  w_down[e] @ gelu(w_up[e] @ (weight * h[t]))`` (the exact gelu; the
     weight scales what goes INTO the expert, not what comes out).  ``w_up [experts, ff, d]``, ``w_down [experts, d, ff]`` in ``h``'s type,
     ``out`` float32 ``[n, d]``.  ``gated``: ``out[t] += sum_e weight * w_down[e] @ (silu(gate[e] @ h[t]) * (up[e] @ h[t]))``
     with ``w_up [experts, 2 * ff, d]`` holding in turns 16 rows of the gate matrix and the 16 up rows that meet them
     (``gated_rows`` lays them out so); ``shared [n, d]`` (with ``shared_gate [n]`` float32, or ones) is added beside;
-    ``fresh``: ``out`` is written, not added to (it need not hold anything)."""
+    ``fresh``: ``out`` is written, not added to (it need not hold anything).  ``identity``: ``ids`` may name ``experts +
+    identity`` experts, of which the last ``identity`` have no matrices: their output is ``weight * h[t]`` (gated form only)."""
     _gpu(h, ids, wts, w_up, w_down, out, shared, shared_gate)
     _rows(h, "moe input")
     for t, what in ((h, "moe input"), (ids, "moe ids"), (wts, "moe weights"), (w_up, "moe up"), (w_down, "moe down"), (out, "moe out")):
@@ -1232,6 +1254,9 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: tor
         raise KernelError(f"moe_experts: the width {d} and the experts' {ff} must be multiples of {per} ({16 if gated else per} for the experts')")
     if fresh and not gated:
         raise KernelError("moe_experts: only the gated form writes its output afresh")
+    identity = int(identity)
+    if identity < 0 or (identity and not gated) or experts + identity > 1024:
+        raise KernelError("moe_experts: identity experts go with gated experts, and all together are at most 1024")
     if shared is not None:
         _contig(shared, "shared expert rows")
         if not gated or shared.shape != (n, d) or shared.dtype != h.dtype:
@@ -1247,7 +1272,7 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: tor
     y = torch.empty((total, d), dtype=torch.float32, device=h.device) if (top > 1 or gated) else None
     _check(lib.lcu_moe_experts(_ptr(h), _type(h, "moe input"), _ptr(ids), _ptr(wts), _ptr(ints), max_tiles, _ptr(w_up),
                                _ptr(w_down), _ptr(act), _ptr(y), _ptr(out), n, d, ff, experts, top, int(bool(gated)),
-                               _ptr(shared), _ptr(shared_gate if shared is not None else None), int(bool(fresh)), _stream()),
+                               _ptr(shared), _ptr(shared_gate if shared is not None else None), int(bool(fresh)), identity, _stream()),
            "moe_experts")
     return out
 
@@ -1507,4 +1532,144 @@ def rglru(rows: torch.Tensor, y_off: int, x_off: int, bias: Optional[torch.Tenso
                          _ptr(scratch[0]), _ptr(scratch[1]), _ptr(scratch[2]), _ptr(out), _type(out, "rglru out"), _ptr(step.q_start),
                          _ptr(step.ctx_len), _ptr(step.req_of_token), _ptr(step.state_slot), n, step.n_req, width, blocks, taps,
                          _stream()), "rglru")
+    return out
+
+
+# ------------------------------------------------------------------ a short convolution over time with its state
+
+
+def _slot_state(state: torch.Tensor, shape, what: str, step) -> int:
+    """Checks a per-request state ``[slots, *shape]`` float32 whose slots may lie apart (a view into a wider state) and
+    returns the distance between two slots in elements."""
+    if state.dtype != torch.float32 or state.dim() != len(shape) + 1 or tuple(state.shape[1:]) != tuple(shape) \
+            or not state[0].is_contiguous():
+        raise KernelError(f"{what}: state must be float32 [slots, {', '.join(str(x) for x in shape)}] with every slot contiguous, "
+                          f"got {state.dtype} {tuple(state.shape)}")
+    if max(step.state_slots, default=0) >= state.shape[0]:
+        raise KernelError(f"{what}: a request's slot lies outside the state")
+    return int(state.stride(0))
+
+
+CONV_ACTIVATIONS = {None: 0, "none": 0, "silu": 1}
+
+
+def causal_conv(rows: torch.Tensor, offset: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
+                step, out_dtype: torch.dtype, activation: Optional[str] = None) -> torch.Tensor:
+    """A causal convolution over time on the ``channels`` columns of ``rows [n, *]`` from ``offset`` on: ``y[t] = act(bias + sum_j
+    weight[:, j] * x[t - taps + 1 + j])`` with ``weight [channels, taps]`` float32 (the last column is the current token's)
+    and places before a request's position 0 counting as zeros.  ``state [slots, taps - 1, channels]`` float32 holds every
+    request's last ``taps - 1`` inputs, is read for the places before the step and moved on by the step's rows (not used
+    with one tap).  Returns ``[n, channels]`` in ``out_dtype``; sums are 32-bit."""
+    _gpu(rows, weight, bias, state)
+    _rows(rows, "conv rows")
+    if rows.stride(1) != 1:
+        raise KernelError("causal_conv: the rows' columns must be contiguous")
+    if weight.dim() != 2 or weight.dtype != torch.float32 or not weight.is_contiguous():
+        raise KernelError("causal_conv: the weight must be contiguous float32 [channels, taps]")
+    channels, taps = weight.shape
+    if not 1 <= taps <= 16:
+        raise KernelError(f"causal_conv: {taps} taps are not supported (1 to 16)")
+    if offset < 0 or offset + channels > rows.shape[1]:
+        raise KernelError(f"causal_conv: the channels lie outside the rows' {rows.shape[1]} columns")
+    _f32_vec(bias, "conv bias", channels)
+    if activation not in CONV_ACTIVATIONS:
+        raise KernelError(f"causal_conv: no activation {activation!r}")
+    n = rows.shape[0]
+    if n != step.n or n > 65535:
+        raise KernelError("causal_conv: the rows are not the step's (or more than 65535)")
+    slot_stride = 0
+    if taps > 1:
+        if state is None:
+            raise KernelError("causal_conv: a convolution of several taps needs its state")
+        slot_stride = _slot_state(state, (taps - 1, channels), "causal_conv", step)
+    out = torch.empty((n, channels), dtype=out_dtype, device=rows.device)
+    lib = build.load("causal_conv")
+    _check(lib.lcu_causal_conv(_ptr(rows), _type(rows, "conv rows"), rows.stride(0), int(offset), _ptr(weight), _ptr(bias),
+                               _ptr(state if taps > 1 else None), ctypes.c_longlong(slot_stride), _ptr(out), _type(out, "conv out"),
+                               out.stride(0), _ptr(step.req_of_token), _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot),
+                               n, step.n_req, channels, taps, CONV_ACTIVATIONS[activation], int(step.decode_only and n == step.n_req),
+                               _stream()), "causal_conv")
+    return out
+
+
+# ------------------------------------------------------------------ the selective scan of a state-space mixer
+
+
+def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, bc: torch.Tensor, a: torch.Tensor, d: torch.Tensor,
+                   z: torch.Tensor, state: torch.Tensor, step) -> torch.Tensor:
+    """``S[c, n] <- exp(dt_c a[c, n]) S[c, n] + dt_c x_c B_n``, ``y_c = sum_n S[c, n] C_n + d_c x_c``, ``out = y * silu(z)`` over
+    the step's rows, request by request from each request's state (``state [slots, channels, states]`` float32, taken as
+    zero at a request's position 0 and left as the step's last token makes it).  ``x [n, channels]`` (its type is the
+    result's), ``dt_raw [n, channels]`` float32 with ``dt = softplus(dt_raw + dt_bias)``, ``bc [n, 2 * states]`` float32
+    holding B then C, ``a [channels, states]`` (negative numbers), ``d [channels]``, ``z [n, channels]`` float32 (rows may
+    be views with a stride)."""
+    _gpu(x, dt_raw, dt_bias, bc, a, d, z, state)
+    for t, what in ((x, "scan x"), (dt_raw, "scan dt"), (bc, "scan B and C"), (z, "scan z")):
+        _rows(t, what)
+        if t.stride(1) != 1:
+            raise KernelError(f"selective_scan: the columns of {what} must be contiguous")
+    n, channels = x.shape
+    if a.dim() != 2 or a.shape[0] != channels or a.dtype != torch.float32 or not a.is_contiguous():
+        raise KernelError(f"selective_scan: a must be contiguous float32 [{channels}, states]")
+    states = a.shape[1]
+    if states > 256:
+        raise KernelError(f"selective_scan: {states} states a channel are not supported (at most 256)")
+    if dt_raw.shape != (n, channels) or z.shape != (n, channels) or bc.shape != (n, 2 * states) \
+            or dt_raw.dtype != torch.float32 or z.dtype != torch.float32 or bc.dtype != torch.float32:
+        raise KernelError("selective_scan: dt and z must be float32 [n, channels] and B, C float32 [n, 2 * states]")
+    _f32_vec(dt_bias, "scan dt bias", channels); _f32_vec(d, "scan d", channels)
+    if n != step.n:
+        raise KernelError("selective_scan: the rows are not the step's")
+    slot_stride = _slot_state(state, (channels, states), "selective_scan", step)
+    out = torch.empty((n, channels), dtype=x.dtype, device=x.device)
+    lib = build.load("selective_scan")
+    _check(lib.lcu_selective_scan(_ptr(x), _type(x, "scan x"), x.stride(0), _ptr(dt_raw), dt_raw.stride(0), _ptr(dt_bias), _ptr(bc),
+                                  bc.stride(0), _ptr(a), _ptr(d), _ptr(z), z.stride(0), _ptr(state), ctypes.c_longlong(slot_stride),
+                                  _ptr(out), out.stride(0), _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot), n,
+                                  step.n_req, channels, states, _stream()), "selective_scan")
+    return out
+
+
+# ------------------------------------------------------------------ the gated delta rule
+
+
+def gated_delta_rule(qkv: torch.Tensor, rows: torch.Tensor, off_a: int, off_b: int, off_g: int, a_log: torch.Tensor,
+                     dt_bias: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, step, heads: int, qk_heads: int,
+                     key_dim: int, value_dim: int, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``S <- g S``, ``u = beta (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q`` per head over the step's rows, request by
+    request from each request's state (``state [slots, heads, key_dim, value_dim]`` float32, taken as zero at a request's
+    position 0).  ``qkv [n, 2 * qk_heads * key_dim + heads * value_dim]`` float32 holds q, k and v behind their
+    convolutions and activations; q and k are made unit vectors per head here (q also times ``key_dim ** -0.5``), and
+    value head ``h`` uses query/key head ``h // (heads / qk_heads)``.  ``rows [n, *]`` float32 holds, at the columns
+    ``off_a``, ``off_b`` (``heads`` each) and ``off_g`` (``heads * value_dim``), the projections that give ``g =
+    exp(-exp(a_log) softplus(a + dt_bias))``, ``beta = sigmoid(b)`` and the output's gate.  Returns each head's ``o``
+    divided by its root mean square (``eps``), times ``weight [value_dim]``, times ``silu(gate)``, ``[n, heads *
+    value_dim]`` in ``out_dtype``."""
+    _gpu(qkv, rows, a_log, dt_bias, weight, state)
+    _rows(qkv, "gated delta q, k, v"); _contig(qkv, "gated delta q, k, v"); _rows(rows, "gated delta rows")
+    n = qkv.shape[0]
+    if heads % qk_heads:
+        raise KernelError(f"gated_delta_rule: {heads} heads are no multiple of {qk_heads} query/key heads")
+    hv = heads * value_dim
+    if qkv.dtype != torch.float32 or qkv.shape[1] != 2 * qk_heads * key_dim + hv:
+        raise KernelError(f"gated_delta_rule: q, k, v must be float32 [n, {2 * qk_heads * key_dim + hv}], got {qkv.dtype} {tuple(qkv.shape)}")
+    if rows.dtype != torch.float32 or rows.shape[0] != n or rows.stride(1) != 1:
+        raise KernelError("gated_delta_rule: the rows must be float32 [n, *] with contiguous columns")
+    for name, off, width in (("a", off_a, heads), ("b", off_b, heads), ("g", off_g, hv)):
+        if off < 0 or off + width > rows.shape[1]:
+            raise KernelError(f"gated_delta_rule: the columns of {name!r} lie outside the rows' {rows.shape[1]} columns")
+    _f32_vec(a_log, "gated delta A_log", heads); _f32_vec(dt_bias, "gated delta dt_bias", heads)
+    _f32_vec(weight, "gated delta norm weight", value_dim)
+    if n != step.n:
+        raise KernelError("gated_delta_rule: the rows are not the step's")
+    slot_stride = _slot_state(state, (heads, key_dim, value_dim), "gated_delta_rule", step)
+    prep = torch.empty((n, heads, 5, key_dim), dtype=torch.float32, device=qkv.device)
+    vb = torch.empty((n, hv), dtype=torch.float32, device=qkv.device)
+    o = torch.empty((n, hv), dtype=torch.float32, device=qkv.device)
+    out = torch.empty((n, hv), dtype=out_dtype, device=qkv.device)
+    lib = build.load("delta_rule")
+    _check(lib.lcu_gated_delta_rule(_ptr(qkv), _ptr(rows), rows.stride(0), int(off_a), int(off_b), int(off_g), _ptr(a_log), _ptr(dt_bias),
+                                    _ptr(weight), _ptr(prep), _ptr(vb), _ptr(o), _ptr(state), ctypes.c_longlong(slot_stride), _ptr(out),
+                                    _type(out, "gated delta out"), _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot), n,
+                                    step.n_req, heads, qk_heads, key_dim, value_dim, ctypes.c_float(eps), _stream()), "gated_delta_rule")
     return out

@@ -1,3 +1,3 @@
 """Architectures: each module turns its typed configuration into a ModelSpec and
 registers itself under the name that config.json's ``architectures`` holds."""
-from . import divasun, llama, lozezen, ralepel  # noqa: F401
+from . import divasun, llama, lozezen, mufotar, ralepel  # noqa: F401

@@ -113,7 +113,8 @@ register_part("block", "prenorm", PreNormBlock)
 
 class ParallelBlock(Part):
     """``x += mixer(c1(norm1(x))) + ffn(c2(norm2(x)))``: two norms of the same ``x``, one sum.  The feed-forward
-    (with its norm) may be missing.
+    (with its norm) may be missing.  ``shared_norm``: there is one norm, and the feed-forward reads what the mixer reads:
+    ``x += mixer(c1(norm1(x))) + ffn(c1(norm1(x)))``.
 
     ``conv_taps > 0``: what each branch reads, ``h``, is first replaced by ``h + conv(h)``, a causal convolution
     over time on each channel with a weight ``[width, taps]`` and no bias (``conv_tensors`` names the two):
@@ -124,8 +125,11 @@ class ParallelBlock(Part):
     residual stream (``pending``)."""
 
     def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, norm2: Optional[PartSpec] = None,
-                 ffn: Optional[PartSpec] = None, conv_taps: int = 0, conv_tensors=("conv1", "conv2")):
-        if (norm2 is None) != (ffn is None):
+                 ffn: Optional[PartSpec] = None, conv_taps: int = 0, conv_tensors=("conv1", "conv2"), shared_norm: bool = False):
+        self.shared_norm = bool(shared_norm)
+        if self.shared_norm and norm2 is not None:
+            raise ValueError("parallel block: with a shared norm there is no second norm")
+        if not self.shared_norm and (norm2 is None) != (ffn is None):
             raise ValueError("parallel block: the second norm and the feed-forward come together or not at all")
         self.hidden_size, self.taps = int(hidden_size), int(conv_taps or 0)
         if self.taps > 16:
@@ -136,7 +140,7 @@ class ParallelBlock(Part):
         self.mixer = make_part("mixer", mixer)
         self.norm2 = make_part("norm", norm2) if norm2 is not None else None
         self.ffn = make_part("ffn", ffn) if ffn is not None else None
-        self.sets = 2 if self.ffn is not None else 1
+        self.sets = 2 if self.norm2 is not None else 1             # how many normed copies of a row there are
         self.graph_safe = all(p.graph_safe for _, p in self._children())
         # two layer norms of the same row are one kernel
         self._pair = isinstance(self.norm1, LayerNorm) and (self.norm2 is None or (isinstance(self.norm2, LayerNorm)
@@ -201,7 +205,7 @@ class ParallelBlock(Part):
             h = ops.norm_conv_single(x, pending, [p.weight for p in norms], [p.bias for p in norms], self.norm1.eps,
                                      self.conv_weight, state, torch.empty((self.sets, n, d), dtype=self.dtype, device=x.device), step)
             out = self.mixer.forward(h[0], step, cache, out_dtype=torch.float32)
-            return self.ffn.forward(h[1], add_to=out) if self.ffn is not None else out
+            return self.ffn.forward(h[self.sets - 1], add_to=out) if self.ffn is not None else out
         h = torch.empty((self.sets, n, d), dtype=mid, device=x.device)
         if self._pair:
             two = self.norm2 is not None
@@ -218,7 +222,7 @@ class ParallelBlock(Part):
             h = ops.short_conv(h, self.conv_weight, state, torch.empty((self.sets, n, d), dtype=self.dtype, device=x.device), step)
         out = self.mixer.forward(h[0], step, cache, out_dtype=torch.float32)
         if self.ffn is not None:
-            out = self.ffn.forward(h[1], add_to=out)
+            out = self.ffn.forward(h[self.sets - 1], add_to=out)
         return out
 
 

@@ -1,4 +1,4 @@
-"""The dense feed-forward: ``down(gate * sigmoid(gate) * up)``.
+"""The dense gated feed-forward: ``down(act(gate) * up)``, ``act`` silu (``gate * sigmoid(gate)``) unless a layout says otherwise.
 
 gate and up projections as one matrix product (gate rows first, the layout of the
 reference's fused tensor, llama.cu/src/model/mod.rs:140-147), the activation of
@@ -24,8 +24,15 @@ class SwiGLU(Part):
     # the tensors' names under the part's own; ``names`` replaces any
     NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
-    def __init__(self, hidden_size: int, intermediate_size: int, names=None):
+    def __init__(self, hidden_size: int, intermediate_size: int, names=None, activation: str = "silu"):
+        """``activation``: what the gate passes through, ``silu`` or ``gelu_tanh`` (the tanh form of gelu).  The products
+        with the activation in their epilogue are written for silu; another activation runs product, activation
+        kernel, product."""
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        if activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"feed-forward: no activation {activation!r}; known: {sorted(ops.GATE_ACTIVATIONS)}")
+        self.activation = str(activation)
+        self.silu = self.activation == "silu"
         self.names = dict(self.NAMES, **(names or {}))
         self.w_gate_up = self.w_down = None
 
@@ -63,7 +70,7 @@ class SwiGLU(Part):
     def takes_scaled_rows(self, n_rows: int) -> bool:
         """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
         plain rows: the factor then goes into the first product's epilogue."""
-        if self.dtype != torch.bfloat16:
+        if self.dtype != torch.bfloat16 or not self.silu:
             return False
         if n_rows <= min(ops.ADD_NORM_MAX_ROWS, skinny_row_limit(self.w_gate_up)) and skinny_takes(n_rows, self.w_gate_up):
             return True
@@ -76,8 +83,21 @@ class SwiGLU(Part):
     # forward(..., planes_ok=True) may return the branch's output as float32 planes of partial sums
     ends_in_planes = True
 
-    def forward(self, h, into=None, planes_ok=False):
-        if isinstance(h, ScaledRows) and mid_swiglu_takes(h.rows.shape[0], self.w_gate_up) and ops.mid_supported(h.rows, self.w_gate_up.plain):
+    def forward(self, h, into=None, planes_ok=False, add_to=None):
+        """``add_to``: float32 ``[n, d]`` that takes the output in (and is returned): the rows of another branch that
+        is added to the stream together with this one."""
+        if add_to is not None:
+            if isinstance(h, ScaledRows) or into is not None:
+                raise ops.KernelError("feed-forward: an output that is added to another branch's takes plain rows and ends in no norm")
+            return ops.scaled_sum(add_to, self._forward(h, out_dtype=torch.float32), 1.0)
+        return self._forward(h, into, planes_ok)
+
+    def _forward(self, h, into=None, planes_ok=False, out_dtype=None):
+        if not self.silu:
+            if isinstance(h, ScaledRows):
+                raise ops.KernelError("feed-forward: rows that wait for their normalisation go with silu only")
+            act = ops.swiglu(linear(h, self.w_gate_up, out_dtype=self.dtype), activation=self.activation)
+        elif isinstance(h, ScaledRows) and mid_swiglu_takes(h.rows.shape[0], self.w_gate_up) and ops.mid_supported(h.rows, self.w_gate_up.plain):
             act = linear_swiglu_mid(h, self.w_gate_up)
         elif isinstance(h, ScaledRows):
             if not ops.skinny_supported(h.rows, self.w_gate_up.plain, self.dtype):
@@ -95,6 +115,8 @@ class SwiGLU(Part):
             act = ops.swiglu(gu)
         if act.shape[1] != self.intermediate_size:
             act = act[:, :self.intermediate_size]      # without what the rows of zeros gave
+        if out_dtype is not None:
+            return linear(act, self.w_down, out_dtype=out_dtype)
         if planes_ok and act.dtype == torch.bfloat16 and mid_takes(act.shape[0], self.w_down):
             # from 12 rows on the product cut over K and the norm kernel that adds its planes are faster
             # than the weight-streaming product with that norm in its epilogue (30 against 35 us)

@@ -44,11 +44,14 @@ class TokenEmbedding(Part):
 class OutputHead(Part):
     graph_safe = True
 
-    """``logits = y @ W.T``; ``tied``: W is the embedding table."""
+    """``logits = y @ W.T``; ``tied``: W is the embedding table.  ``softcap`` c > 0: ``logits <- c tanh(logits / c)``."""
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, tensor: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, tensor: str = "weight", softcap: float = 0.0):
         self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)
         self.tensor = str(tensor)
+        self.softcap = float(softcap or 0.0)
+        if self.softcap < 0:
+            raise ValueError(f"output matrix: the cap on the logits {softcap} must be positive (or 0 for none)")
         self.weight = None
 
     def tensors(self):
@@ -68,8 +71,10 @@ class OutputHead(Part):
 
     def forward(self, y) -> torch.Tensor:
         if isinstance(y, ScaledRows):
-            return linear_scaled(y, self.weight, out_dtype=torch.float32)
-        return linear(y, self.weight, out_dtype=torch.float32)
+            logits = linear_scaled(y, self.weight, out_dtype=torch.float32)
+        else:
+            logits = linear(y, self.weight, out_dtype=torch.float32)
+        return ops.softcap(logits, self.softcap) if self.softcap else logits
 
 
 register_part("embedding", "tokens", TokenEmbedding)

@@ -84,18 +84,35 @@ class GatedMoE(Part):
               + sigmoid(w_sg . h) * shared(h)          (``shared``: a dense gated feed-forward that every token uses)
 
     The weight scales what comes OUT of an expert.  The shared expert's gate is one more row of the router's matrix, so
-    its logit is made by the routing kernel, in 32-bit.  The output is 32-bit rows."""
+    its logit is made by the routing kernel, in 32-bit.  The output is 32-bit rows.
+
+    ``scoring="softmax_all"``: the scores are ``s = softmax(z)`` over all experts, the ``top`` largest of ``s + correction``
+    are chosen (``correction``: a tensor ``[experts]`` that moves the choice and nothing else), and the weights are the chosen
+    ``s`` divided by their sum + 1e-20.  ``identity``: so many more outputs of the router, behind the experts', stand for
+    identity experts, which have no tensors and whose output is the input itself (times the weight).
+    ``shared_gated=False``: the shared expert is added as it is, without a gate.  ``forward(h, add_to=)`` adds the output
+    into 32-bit rows that hold another branch's output already."""
     graph_safe = True
 
     NAMES = {"router": "router", "router_bias": "router.b", "gate": "e{}.gate", "up": "e{}.up", "down": "e{}.down",
-             "shared_gate": "shared.gate", "shared_up": "shared.up", "shared_down": "shared.down", "shared_sg": "shared.sg"}
+             "shared_gate": "shared.gate", "shared_up": "shared.up", "shared_down": "shared.down", "shared_sg": "shared.sg",
+             "correction": "correction"}
+    SCORINGS = ("softmax_chosen", "softmax_all")
 
     def __init__(self, hidden_size: int, expert_size: int, experts: int, top: int, shared_size: Optional[int] = None,
-                 router_bias: bool = True, names: Optional[Dict[str, str]] = None):
+                 router_bias: bool = True, names: Optional[Dict[str, str]] = None, scoring: str = "softmax_chosen",
+                 correction: bool = False, identity: int = 0, shared_gated: bool = True):
         self.hidden_size, self.expert_size = int(hidden_size), int(expert_size)
-        self.experts, self.top = int(experts), int(top)
-        if not 1 <= self.top <= self.experts or self.experts > 1024:
-            raise ValueError(f"moe: top {top} of {experts} experts is not supported (1 <= top <= experts <= 1024)")
+        self.experts, self.top, self.identity = int(experts), int(top), int(identity)
+        self.outputs = self.experts + self.identity          # what the router chooses among
+        if not 1 <= self.top <= self.outputs or self.outputs > 1024 or self.experts < 1 or self.identity < 0:
+            raise ValueError(f"moe: top {top} of {experts} experts and {identity} identity experts is not supported "
+                             f"(1 <= top <= experts + identity <= 1024)")
+        if scoring not in self.SCORINGS:
+            raise ValueError(f"moe: no scoring {scoring!r}; known: {list(self.SCORINGS)}")
+        if correction and scoring != "softmax_all":
+            raise ValueError("moe: a correction of the choice goes with scores over all experts")
+        self.scoring, self.correction, self.shared_gated = scoring, bool(correction), bool(shared_gated)
         self.names = dict(self.NAMES, **(names or {}))
         self.router_bias = bool(router_bias)
         self.shared = None
@@ -111,15 +128,18 @@ class GatedMoE(Part):
 
     def tensors(self) -> Dict[str, TensorSpec]:
         d, ff, nm = self.hidden_size, self.expert_size, self.names
-        t = {nm["router"]: TensorSpec((self.experts, d))}
+        t = {nm["router"]: TensorSpec((self.outputs, d))}
         if self.router_bias:
-            t[nm["router_bias"]] = TensorSpec((self.experts,))
+            t[nm["router_bias"]] = TensorSpec((self.outputs,))
+        if self.correction:
+            t[nm["correction"]] = TensorSpec((self.outputs,))
         for key, shape in (("gate", (ff, d)), ("up", (ff, d)), ("down", (d, ff))):
             for n in self._each(key):
                 t[n] = TensorSpec(shape)
         if self.shared is not None:
             t.update(self.shared.tensors())
-            t[nm["shared_sg"]] = TensorSpec((1, d))
+            if self.shared_gated:
+                t[nm["shared_sg"]] = TensorSpec((1, d))
         return t
 
     def fused_groups(self, dtype, device):
@@ -128,9 +148,14 @@ class GatedMoE(Part):
 
     def load(self, tensors, build: BuildContext) -> None:
         d, ff, n, nm = self.hidden_size, self.expert_size, self.experts, self.names
-        rows = [tensors[nm["router"]].float()] + ([tensors[nm["shared_sg"]].float().view(1, d)] if self.shared is not None else [])
+        self.gates = 1 if (self.shared is not None and self.shared_gated) else 0
+        rows = [tensors[nm["router"]].float()] + ([tensors[nm["shared_sg"]].float().view(1, d)] if self.gates else [])
         self.router = torch.cat(rows).contiguous()                          # the router, and the shared expert's gate, are 32-bit
         self.bias = tensors[nm["router_bias"]].float().contiguous() if self.router_bias else None
+        if self.correction:
+            if self.bias is not None:
+                raise ValueError("moe: a bias on the logits and a correction of the choice together are not supported")
+            self.bias = tensors[nm["correction"]].float().contiguous()
         gate = fused_rows([tensors[k] for k in self._each("gate")]).view(n, ff, d)
         up = fused_rows([tensors[k] for k in self._each("up")]).view(n, ff, d)
         self.w_down = fused_rows([tensors[k] for k in self._each("down")]).view(n, d, ff)
@@ -146,15 +171,19 @@ class GatedMoE(Part):
             self.shared.load(tensors, build)
         self.dtype = build.dtype
 
-    def forward(self, h):
-        routed = ops.moe_route(h, self.router, self.top, bias=self.bias, softmax_chosen=True, extra=1 if self.shared is not None else 0)
+    def forward(self, h, add_to: Optional[torch.Tensor] = None):
+        """``add_to``: float32 ``[n, d]`` that takes the output in (and is returned); without it the output is new rows."""
+        over_all = self.scoring == "softmax_all"
+        routed = ops.moe_route(h, self.router, self.top, bias=self.bias, softmax_chosen=not over_all, softmax_all=over_all,
+                               extra=self.gates)
         ids, wts = routed[0], routed[1]
-        out = torch.empty((h.shape[0], self.hidden_size), dtype=torch.float32, device=h.device)
+        fresh = add_to is None
+        out = add_to if not fresh else torch.empty((h.shape[0], self.hidden_size), dtype=torch.float32, device=h.device)
         if self.shared is not None:
             ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True, shared=self.shared.forward(h),
-                            shared_gate=routed[2], fresh=True)
+                            shared_gate=routed[2] if self.gates else None, fresh=fresh, identity=self.identity)
         else:
-            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True, fresh=True)
+            ops.moe_experts(h, ids, wts, self.w_gate_up, self.w_down, out, gated=True, fresh=fresh, identity=self.identity)
         return out
 
 
