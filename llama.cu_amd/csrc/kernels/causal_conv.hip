@@ -78,12 +78,13 @@ causal_conv_single_kernel(const TI *__restrict__ x, int x_stride, int x_off, con
     const bool fresh = ctx_len[r] == 1;
     float *st = state + (size_t)state_slot[r] * slot_stride + c;
     const float cur = to_f32(x[(size_t)r * x_stride + x_off + c]);
-    float acc = (bias ? bias[c] : 0.f) + w[(size_t)c * taps + taps - 1] * cur;
-    for (int i = 0; i < taps - 1; ++i) {
+    float acc = bias ? bias[c] : 0.f;
+    for (int i = 0; i < taps - 1; ++i) {                 // (the taps in the order of the kernel for portions: the same bits)
         const float v = fresh ? 0.f : st[(size_t)i * channels];
         acc += w[(size_t)c * taps + i] * v;
         if (i > 0) st[(size_t)(i - 1) * channels] = v;
     }
+    acc += w[(size_t)c * taps + taps - 1] * cur;
     if (taps > 1) st[(size_t)(taps - 2) * channels] = cur;
     out[(size_t)r * out_stride + c] = from_f32<TO>(conv_act(acc, act));
 }

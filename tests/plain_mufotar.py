@@ -84,8 +84,9 @@ def softmax_attention(h, W, pre, m, eps):
     q = rms_div(q, eps) * W[pre + "q.norm"]
     k = rms_div(k, eps) * W[pre + "k.norm"]
     pos = np.arange(T, dtype=np.float64)
-    q = rotate_half_split(q, pos, m["rot"]["base"], m["rot"]["dims"])
-    k = rotate_half_split(k, pos, m["rot"]["base"], m["rot"]["dims"])
+    if m.get("rot"):
+        q = rotate_half_split(q, pos, m["rot"]["base"], m["rot"]["dims"])
+        k = rotate_half_split(k, pos, m["rot"]["base"], m["rot"]["dims"])
     out = np.zeros((T, H, vdim))
     mask = np.tril(np.ones((T, T), dtype=bool))
     for hd in range(H):
