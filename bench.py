@@ -417,8 +417,37 @@ def ralepel_config(z, positions):
                                     "max_positions": positions})
 
 
+def mufotar_config(z, positions):
+    """The gated delta rule three times and the side-by-side mixer (attention with half of each head rotated beside a
+    selective scan over ``width`` channels of 16 states) once, in turn; the first layer with the dense feed-forward of the
+    Llama model beside it, the others with a mixture of experts whose active weights (the chosen experts and the shared
+    one) are about as many, two identity experts behind the experts; the last layer runs the parts of the layer four before it
+    once more."""
+    from llama_cu_amd.config import MufotarConfig
+    inter = (z["top"] * 2 * z["ff"] // 3 + 127) // 128 * 128
+    shared = inter // 4 // 64 * 64
+    expert = (inter - shared) // z["top"] // 64 * 64
+    d, h, g, w = z["dim"], z["heads"], z["kv_heads"], z["width"]
+    layers = []
+    for i in range(z["layers"]):
+        if i % 4 == 2:
+            kind = "parallel"
+            m = {"left": {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "rot": {"dims": d // 2, "base": 1000000.0}},
+                 "right": {"inner": w, "state": 16, "dt_rank": w // 16, "conv": 4}, "left_scale": 1.0, "right_scale": 0.5}
+        else:
+            kind, m = "delta", {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "conv": 4}
+        mlp = {"kind": "dense", "ff": inter} if i == 0 else \
+            {"kind": "moe", "router": {"experts": z["experts"], "identity": 2, "top": z["top"]}, "expert": {"ff": expert}, "shared": {"ff": shared}}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    if len(layers) > 4:
+        layers[-1] = dict(layers[-5], weights_of=len(layers) - 5)
+    return MufotarConfig.from_dict({"architecture": "Mufotar", "vocab": z["vocab"], "width": w, "layers": layers, "norm": {"eps": 1e-5},
+                                    "logit_softcap": 30.0, "max_positions": positions})
+
+
 DESIGN_CONFIGS = {"divasun": lambda z, p: divasun_config(z, p), "llama": lambda z, p: llama_like(z, p),
-                  "lozezen": lambda z, p: lozezen_config(z, p), "ralepel": lambda z, p: ralepel_config(z, p)}
+                  "lozezen": lambda z, p: lozezen_config(z, p), "ralepel": lambda z, p: ralepel_config(z, p),
+                  "mufotar": lambda z, p: mufotar_config(z, p)}
 
 
 def llama_like(z, positions):
@@ -545,10 +574,10 @@ def main() -> int:
                          "decode while a prompt of 16 tokens arrives every second step (host time and the GPU's busy "
                          "fraction per kind of step)")
     ap.add_argument("--designs", default="divasun,llama", metavar="NAMES",
-                    help="with --workload designs: which designs are measured side by side, of divasun, lozezen, ralepel and llama "
+                    help="with --workload designs: which designs are measured side by side, of divasun, lozezen, ralepel, mufotar and llama "
                          "(default: divasun,llama)")
     ap.add_argument("--designs-one", metavar="DESIGN:SIZE:WHAT", default=None,
-                    help="with --workload designs, for a profiler: only DESIGN (divasun, lozezen, ralepel or llama) at SIZE (w2048, w4096), and "
+                    help="with --workload designs, for a profiler: only DESIGN (divasun, lozezen, ralepel, mufotar or llama) at SIZE (w2048, w4096), and "
                          "only WHAT: 'prefill' (three steps of 2,048 tokens) or a number of requests that decode ten steps over "
                          "prompts of 512 tokens; steps are launched one kernel at a time, not replayed from graphs")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64, the prefill and the check")
