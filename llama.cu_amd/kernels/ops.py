@@ -1623,10 +1623,13 @@ def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
     slot_stride = _slot_state(state, (channels, states), "selective_scan", step)
     out = torch.empty((n, channels), dtype=x.dtype, device=x.device)
     lib = build.load("selective_scan")
+    # requests that feed many tokens are walked in runs side by side: each run's own sums, then the state it starts from
+    n_long = sum(1 for q in step.q_lens if q >= lib.lcu_selective_scan_long())
+    runs = torch.empty(n_long * lib.lcu_selective_scan_runs() * channels * (states + 1), dtype=torch.float32, device=x.device) if n_long else None
     _check(lib.lcu_selective_scan(_ptr(x), _type(x, "scan x"), x.stride(0), _ptr(dt_raw), dt_raw.stride(0), _ptr(dt_bias), _ptr(bc),
                                   bc.stride(0), _ptr(a), _ptr(d), _ptr(z), z.stride(0), _ptr(state), ctypes.c_longlong(slot_stride),
                                   _ptr(out), out.stride(0), _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot), n,
-                                  step.n_req, channels, states, _stream()), "selective_scan")
+                                  step.n_req, channels, states, _ptr(runs), _stream()), "selective_scan")
     return out
 
 

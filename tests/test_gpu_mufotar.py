@@ -62,8 +62,9 @@ class Feeder:
     tokens and portions of the second, which starts later; slots 2 and 0 of a state that holds other values; with pages,
     a block table of shuffled pages among pages that nobody owns."""
 
-    def __init__(self, lens, page=16, seed=0):
-        self.lens, self.page = lens, page
+    def __init__(self, lens, page=16, seed=0, steps=None):
+        """``steps``: the plan, if not the usual one: [[(request, first token, tokens taken), ...], ...]."""
+        self.lens, self.page, self.steps = lens, page, steps
         rng = random.Random(seed)
         need = [(n + page - 1) // page for n in lens]
         order = list(range(sum(need) + 3))
@@ -79,7 +80,9 @@ class Feeder:
         self.bt = bt.cuda()
 
     def plan(self):
-        """[(request, tokens taken)] per step."""
+        """[(request, first token, tokens taken)] per step."""
+        if self.steps is not None:
+            return self.steps
         l0, l1 = self.lens
         steps, a, b = [], 0, 0
         sizes0, sizes1 = [5, 1, 2, 7, 1, 1, 3, 16, 2, 1], [1, 2, 1, 4, 9, 1, 2]
@@ -194,6 +197,26 @@ def test_the_selective_scan_against_its_recurrence(dtype, inner, states, rank, t
     for r in range(2):
         want = P.selective_scan(f64(rows[r].float()), wn, "p.", right(inner, states, rank, taps))
         assert_close(got[r], want, 1e-5 if dtype == "float32" else 4e-2, f"request {r}")
+
+
+@pytest.mark.parametrize("inner,states,rank,taps", [(72, 6, 5, 3), (256, 16, 8, 4)])
+def test_the_selective_scan_walks_long_portions_in_runs(inner, states, rank, taps):
+    """Portions of 512 tokens and more are walked in runs side by side and chained: a long portion from the start beside a
+    short request, a second long one that goes on from the first's state, then single tokens."""
+    d = 48
+    cfg = config(16, d, [{"type": "parallel", "mixer": parallel(left(1, 1, 8, 8, 0.3), right(inner, states, rank, taps)), "mlp": None}], 1e-5)
+    w = {k[len("l0.mix.right."):]: v for k, v in random_weights(cfg, 7).items() if k.startswith("l0.mix.right.")}
+    part = built("mixer", "selective_scan", {"hidden_size": d, "inner": inner, "states": states, "dt_rank": rank, "taps": taps}, w, torch.float32)
+    lens = [1303, 530]
+    rows = [rnd(n, d, seed=30 + r) for r, n in enumerate(lens)]
+    cache = part.cache_need().allocate(-1, 0, 0, 3, torch.float32, torch.device("cuda"))
+    cache.state.normal_(0.0, 7.0)
+    steps = [[(0, 0, 600), (1, 0, 7)], [(1, 7, 520), (0, 600, 700)], [(0, 1300, 1), (1, 527, 1)], [(0, 1301, 2), (1, 528, 2)]]
+    got = Feeder(lens, steps=steps).run(lambda step, x: part.forward(x.cuda(), step, cache, out_dtype=torch.float32), rows)
+    wn = {"p." + k: f64(v) for k, v in w.items()}
+    for r in range(2):
+        want = P.selective_scan(f64(rows[r]), wn, "p.", right(inner, states, rank, taps))
+        assert_close(got[r], want, 1e-5, f"request {r}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
