@@ -181,6 +181,27 @@ def test_the_gated_delta_rule_gives_the_same_bits_however_a_prompt_is_cut():
     assert torch.equal(torch.cat(parts), whole)
 
 
+@pytest.mark.parametrize("heads,qk_heads,dk,dv,taps", [(4, 2, 64, 40, 3), (2, 1, 16, 48, 4), (3, 3, 48, 12, 2), (2, 2, 24, 20, 2)])
+def test_the_gated_delta_rule_over_long_portions(heads, qk_heads, dk, dv, taps):
+    """Portions of hundreds of tokens: a long portion from the start beside a short request, a second long one that goes on
+    from the first's state, then single tokens."""
+    d, eps = 56, 1e-5
+    cfg = config(16, d, [{"type": "delta", "mixer": delta(heads, qk_heads, dk, dv, taps), "mlp": None}], eps)
+    w = {k[len("l0.mix."):]: v for k, v in random_weights(cfg, 5).items() if k.startswith("l0.mix.")}
+    part = built("mixer", "gated_delta", {"hidden_size": d, "heads": heads, "qk_heads": qk_heads, "head_dim": dk, "value_dim": dv,
+                                          "taps": taps, "norm_eps": eps}, w, torch.float32)
+    lens = [1303, 530]
+    rows = [rnd(n, d, seed=20 + r) for r, n in enumerate(lens)]
+    cache = part.cache_need().allocate(-1, 0, 0, 3, torch.float32, torch.device("cuda"))
+    cache.state.normal_(0.0, 7.0)
+    steps = [[(0, 0, 600), (1, 0, 7)], [(1, 7, 520), (0, 600, 700)], [(0, 1300, 1), (1, 527, 1)], [(0, 1301, 2), (1, 528, 2)]]
+    got = Feeder(lens, steps=steps).run(lambda step, x: part.forward(x.cuda(), step, cache, out_dtype=torch.float32), rows)
+    wn = {"p." + k: f64(v) for k, v in w.items()}
+    for r in range(2):
+        want = P.gated_delta(f64(rows[r]), wn, "p.", delta(heads, qk_heads, dk, dv, taps), eps)
+        assert_close(got[r], want, 2e-5, f"request {r}")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("inner,states,rank,taps", [(40, 6, 5, 2), (256, 16, 8, 4), (8, 1, 1, 1), (24, 5, 3, 5), (72, 70, 4, 3), (130, 4, 9, 2)])
 def test_the_selective_scan_against_its_recurrence(dtype, inner, states, rank, taps):
