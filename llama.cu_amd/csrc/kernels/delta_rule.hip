@@ -85,7 +85,10 @@ __device__ __forceinline__ float sum_over_groups(float x) {
 template <class T, int DK>
 constexpr int scan_groups() { return DK > 0 && DK % 32 == 0 ? 8 : 4; }
 
-template <class T, int DK>
+// GATED: the gated rule, whose decay g and rate beta are one number each per token and head and whose key is its unit
+// key: S <- g S + u (v - (beta g) (u^T S)) with v the value times beta already.  A token then brings two vectors (u, r) and
+// two numbers (g, beta g) instead of five vectors: prep rows are [u | r | g, beta g, 0, 0], 2 dk + 4 floats.
+template <class T, int DK, bool GATED>
 __global__ void __launch_bounds__(64)
 delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const float *__restrict__ vf, const float *__restrict__ prep,
                   float *__restrict__ state, size_t slot_stride, float *__restrict__ o, const int *__restrict__ q_start,
@@ -96,7 +99,9 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
     if constexpr (DK > 0) {
         constexpr int SCAN_GROUPS = scan_groups<T, DK>(), SCAN_COLS = WAVE / SCAN_GROUPS;
         constexpr int SL = DK / SCAN_GROUPS;                  // key channels of a lane
-        constexpr int PER_LANE = (5 * DK + 63) / 64;
+        constexpr int NV = GATED ? 2 : 5;                     // vectors of a token
+        constexpr int ROW = NV * DK + (GATED ? 4 : 0);        // floats of a token's prep row
+        constexpr int PER_LANE = (ROW + 63) / 64;
         constexpr int TB = DK <= 128 ? 8 : 4;                 // tokens whose vectors are brought in together
         const int g = threadIdx.x / SCAN_COLS, j = blockIdx.z * SCAN_COLS + threadIdx.x % SCAN_COLS;
         const bool live = j < dv;
@@ -105,7 +110,7 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
         // a vector in LDS: the four groups' quarters, each followed by four floats of padding, so that the groups' reads of
         // their quarters (the same offset in each) fall into different banks
         constexpr int SLP = SL + 4, VEC = SCAN_GROUPS * SLP;
-        __shared__ __attribute__((aligned(16))) float vec[2][TB][5 * VEC];
+        __shared__ __attribute__((aligned(16))) float vec[2][TB][NV * VEC + (GATED ? 4 : 0)];
         float S[SL];
 #pragma unroll
         for (int i = 0; i < SL; ++i) S[i] = fresh ? 0.f : col[(size_t)i * dv];
@@ -118,11 +123,11 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
 #pragma unroll
             for (int b = 0; b < TB; ++b) {
                 if (t + b >= t1) break;                       // (a step of one token brings in one token)
-                const float *p = prep + ((size_t)(t + b) * heads + h) * 5 * DK;
+                const float *p = prep + ((size_t)(t + b) * heads + h) * ROW;
 #pragma unroll
                 for (int e = 0; e < PER_LANE; ++e) {
                     const int idx = e * 64 + threadIdx.x;
-                    next[b][e] = idx < 5 * DK ? p[idx] : 0.f;
+                    next[b][e] = idx < ROW ? p[idx] : 0.f;
                 }
                 v_next[b] = vfp ? vfp[(size_t)(t + b) * heads * dv] : to_f32(vp[(size_t)(t + b) * row_stride]);
             }
@@ -138,7 +143,8 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
 #pragma unroll
                 for (int e = 0; e < PER_LANE; ++e) {
                     const int idx = e * 64 + threadIdx.x;
-                    if (idx < 5 * DK) vec[turn][b][idx / DK * VEC + idx % DK / SL * SLP + idx % SL] = next[b][e];
+                    if (idx < NV * DK) vec[turn][b][idx / DK * VEC + idx % DK / SL * SLP + idx % SL] = next[b][e];
+                    else if (GATED && idx < ROW) vec[turn][b][NV * VEC + idx - NV * DK] = next[b][e];
                 }
             }
             __syncthreads();                                  // (the buffer of two turns ago was last read before the barrier of the turn between)
@@ -146,7 +152,8 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
 #pragma unroll
             for (int b = 0; b < TB; ++b) {
                 if (t + b >= t1) break;
-                const float *W = vec[turn][b] + g * SLP, *AU = W + VEC, *U = W + 2 * VEC, *K = W + 3 * VEC, *R = W + 4 * VEC;
+                const float *W = vec[turn][b] + g * SLP, *AU = W + VEC, *U = GATED ? W : W + 2 * VEC, *K = W + 3 * VEC,
+                            *R = GATED ? W + VEC : W + 4 * VEC;
                 // four sums side by side in each pass (added in a fixed order): one chain of SL dependent additions
                 // would be most of a token's time
                 float us4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -154,10 +161,19 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
                 for (int i = 0; i < SL; ++i) us4[i & 3] += U[i] * S[i];
                 const float us = sum_over_groups<SCAN_GROUPS>((us4[0] + us4[1]) + (us4[2] + us4[3]));
                 float acc4[4] = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (GATED) {
+                    const float gd = vec[turn][b][NV * VEC], c = v[b] - vec[turn][b][NV * VEC + 1] * us;
 #pragma unroll
-                for (int i = 0; i < SL; ++i) {
-                    S[i] = W[i] * S[i] - AU[i] * us + K[i] * v[b];
-                    acc4[i & 3] += S[i] * R[i];
+                    for (int i = 0; i < SL; ++i) {
+                        S[i] = gd * S[i] + U[i] * c;
+                        acc4[i & 3] += S[i] * R[i];
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < SL; ++i) {
+                        S[i] = W[i] * S[i] - AU[i] * us + K[i] * v[b];
+                        acc4[i & 3] += S[i] * R[i];
+                    }
                 }
                 const float acc = sum_over_groups<SCAN_GROUPS>((acc4[0] + acc4[1]) + (acc4[2] + acc4[3]));
                 if (live && g == 0) o[(size_t)(t + b) * heads * dv + h * dv + j] = acc;
@@ -176,13 +192,23 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
             for (int i = 0; i < dk; ++i) col[(size_t)i * dv] = 0.f;
         for (int t = t0; t < t1; ++t) {
             const float v = vf ? vf[(size_t)t * heads * dv + h * dv + jj] : to_f32(proj[(size_t)t * row_stride + off_v + h * dv + jj]);
-            const float *p = prep + ((size_t)t * heads + h) * 5 * dk;
+            const float *p = prep + ((size_t)t * heads + h) * (GATED ? 2 * dk + 4 : 5 * dk);
             float us = 0.f, acc = 0.f;
-            for (int i = 0; i < dk; ++i) us += p[2 * dk + i] * col[(size_t)i * dv];
-            for (int i = 0; i < dk; ++i) {
-                const float s = p[i] * col[(size_t)i * dv] - p[dk + i] * us + p[3 * dk + i] * v;
-                if (live) col[(size_t)i * dv] = s;
-                acc += s * p[4 * dk + i];
+            if constexpr (GATED) {
+                for (int i = 0; i < dk; ++i) us += p[i] * col[(size_t)i * dv];
+                const float gd = p[2 * dk], c = v - p[2 * dk + 1] * us;
+                for (int i = 0; i < dk; ++i) {
+                    const float s = gd * col[(size_t)i * dv] + p[i] * c;
+                    if (live) col[(size_t)i * dv] = s;
+                    acc += s * p[dk + i];
+                }
+            } else {
+                for (int i = 0; i < dk; ++i) us += p[2 * dk + i] * col[(size_t)i * dv];
+                for (int i = 0; i < dk; ++i) {
+                    const float s = p[i] * col[(size_t)i * dv] - p[dk + i] * us + p[3 * dk + i] * v;
+                    if (live) col[(size_t)i * dv] = s;
+                    acc += s * p[4 * dk + i];
+                }
             }
             if (live) o[(size_t)t * heads * dv + h * dv + j] = acc;
         }
@@ -207,11 +233,11 @@ delta_out_kernel(const float *__restrict__ o, const T *__restrict__ proj, int ro
 }
 
 // The scan over the step's tokens for every head size it is compiled for.  vf: null, or the values as 32-bit rows.
-template <class T>
+template <class T, bool GATED = false>
 static int delta_scan_launch(const T *proj, int row_stride, int off_v, const float *vf, const float *prep, float *state,
                              size_t slot_stride, float *o, const int *q_start, const int *ctx_len, const int *state_slot,
                              int n_req, int heads, int dk, int dv, hipStream_t stream) {
-#define SCAN(DK) delta_scan_kernel<T, DK><<<dim3(n_req, heads, (dv + (DK ? 64 / scan_groups<T, DK>() : 64) - 1) / (DK ? 64 / scan_groups<T, DK>() : 64)), dim3(64), 0, stream>>>(proj, row_stride, off_v, vf, prep, state, slot_stride, o, q_start, ctx_len, state_slot, heads, dk, dv)
+#define SCAN(DK) delta_scan_kernel<T, DK, GATED><<<dim3(n_req, heads, (dv + (DK ? 64 / scan_groups<T, DK>() : 64) - 1) / (DK ? 64 / scan_groups<T, DK>() : 64)), dim3(64), 0, stream>>>(proj, row_stride, off_v, vf, prep, state, slot_stride, o, q_start, ctx_len, state_slot, heads, dk, dv)
     switch (dk) {
     case 16: SCAN(16); break;
     case 32: SCAN(32); break;
@@ -267,9 +293,10 @@ LCU_API int lcu_delta_rule(const void *proj, int type, int row_stride, int off_r
 // ---------------------------------------------------------------- the gated delta rule
 // One decay and one rate per head and token:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q,  with q and k
 // unit vectors per head (q also times dk^-1/2).  Written out, S <- g S - (beta g k)(k^T S) + k (beta v)^T with S as the
-// token found it: the scan above with the decay g on every key channel, the removal vector beta g k, and the values
-// beta v.  Several value heads may share one query/key head (`group` of them).
-//   prep (parallel over tokens and value heads): the scan's five vectors and the values times beta;
+// token found it, or S <- g S + k (beta v - (beta g)(k^T S)): the scan above in its gated form, which takes per token
+// the unit key, the query, the two numbers g and beta g, and the values beta v.  Several value heads may share one
+// query/key head (`group` of them).
+//   prep (parallel over tokens and value heads): the scan's two vectors and two numbers, and the values times beta;
 //   out  (parallel): o of each head divided by its root mean square, times a weight, times silu(gate).
 // qkv: [n, qk_heads * dk (q) | qk_heads * dk (k) | heads * dv (v)] 32-bit, the projections behind their convolutions
 // and activations.  rows: [n, row_stride] 32-bit holding per head the decay's and the rate's projections at columns
@@ -295,15 +322,12 @@ __global__ void gated_delta_prep_kernel(const float *__restrict__ qkv, const flo
     const float *row = rows + (size_t)t * row_stride;
     const float beta = sigmoidf_(row[off_b + h]);
     const float g = expf(-expf(a_log[h]) * softplus_(row[off_a + h] + dt_bias[h]));
-    float *out = prep + ((size_t)t * heads + h) * 5 * dk;
+    float *out = prep + ((size_t)t * heads + h) * (2 * dk + 4);
     for (int i = threadIdx.x; i < dk; i += blockDim.x) {
-        const float u = k[i] * kf;
-        out[i] = g;
-        out[dk + i] = beta * g * u;
-        out[2 * dk + i] = u;
-        out[3 * dk + i] = u;
-        out[4 * dk + i] = q[i] * qf;
+        out[i] = k[i] * kf;
+        out[dk + i] = q[i] * qf;
     }
+    if (threadIdx.x < 4) out[2 * dk + threadIdx.x] = threadIdx.x == 0 ? g : (threadIdx.x == 1 ? beta * g : 0.f);
     for (int j = threadIdx.x; j < dv; j += blockDim.x) vb[((size_t)t * heads + h) * dv + j] = beta * v[j];
 }
 
@@ -323,7 +347,7 @@ gated_delta_out_kernel(const float *__restrict__ o, const float *__restrict__ ro
     }
 }
 
-// a_log, dt_bias: [heads]; weight: [dv], 32-bit.  prep: scratch [n, heads, 5, dk]; vb, o: scratch [n, heads * dv], 32-bit.
+// a_log, dt_bias: [heads]; weight: [dv], 32-bit.  prep: scratch [n, heads, 2 * dk + 4]; vb, o: scratch [n, heads * dv], 32-bit.
 // state: slot s at state + s * slot_stride, [heads, dk, dv] 32-bit.  out: [n, heads * dv] of out_type.
 LCU_API int lcu_gated_delta_rule(const float *qkv, const float *rows, int row_stride, int off_a, int off_b, int off_g,
                                  const float *a_log, const float *dt_bias, const float *weight, float *prep, float *vb, float *o,
@@ -339,7 +363,7 @@ LCU_API int lcu_gated_delta_rule(const float *qkv, const float *rows, int row_st
     gated_delta_prep_kernel<<<dim3(n, heads), dim3(threads), 0, stream>>>(qkv, rows, row_stride, off_a, off_b, a_log, dt_bias, prep, vb,
                                                                            heads, heads / qk_heads, dk, dv);
     LCU_LAUNCH_CHECK();
-    const int rc = delta_scan_launch<float>(nullptr, 0, 0, vb, prep, state, (size_t)slot_stride, o, q_start, ctx_len, state_slot, n_req,
+    const int rc = delta_scan_launch<float, true>(nullptr, 0, 0, vb, prep, state, (size_t)slot_stride, o, q_start, ctx_len, state_slot, n_req,
                                             heads, dk, dv, stream);
     if (rc != LCU_OK) return rc;
     if (out_type == LCU_F32)

@@ -1666,7 +1666,7 @@ def gated_delta_rule(qkv: torch.Tensor, rows: torch.Tensor, off_a: int, off_b: i
     if n != step.n:
         raise KernelError("gated_delta_rule: the rows are not the step's")
     slot_stride = _slot_state(state, (heads, key_dim, value_dim), "gated_delta_rule", step)
-    prep = torch.empty((n, heads, 5, key_dim), dtype=torch.float32, device=qkv.device)
+    prep = torch.empty((n, heads, 2 * key_dim + 4), dtype=torch.float32, device=qkv.device)     # per token and head: unit key, query, g, beta g
     vb = torch.empty((n, hv), dtype=torch.float32, device=qkv.device)
     o = torch.empty((n, hv), dtype=torch.float32, device=qkv.device)
     out = torch.empty((n, hv), dtype=out_dtype, device=qkv.device)
