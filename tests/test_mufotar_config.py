@@ -127,3 +127,26 @@ def test_routing_chooses_by_the_corrected_scores_and_weighs_by_the_scores():
     W.update({f"m.e{e}.{n}": np.zeros((2, 4)) if n != "down" else np.zeros((4, 2)) for e in range(3) for n in ("gate", "up", "down")})
     out = P.mixture_ff(h, W, "m.", f)
     assert np.allclose(out, wts[0, 0] * h)
+
+
+def test_the_bench_configurations_of_the_design_build_and_hold_the_dense_models_active_weights():
+    """``bench.py --workload designs``: the design's configuration at both sizes reads as a model, the larger run order names
+    a layer twice, and a mixture layer's active feed-forward weights are within a tenth of the dense model's."""
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    twice = 0
+    for z in bench.DESIGN_SIZES.values():
+        cfg = bench.mufotar_config(z, 4096)
+        model = DecoderModel(architecture_of(cfg.to_dict()).build_spec(cfg))
+        assert len(model.spec.run_order) == z["layers"] and model.tensors()
+        twice += len(model.spec.run_order) - len(model.layers)
+        assert {l.type for l in cfg.layers} == {"delta", "parallel"}
+        dense = [l.ff for l in cfg.layers if isinstance(l.ff, int)][0]
+        for layer in cfg.layers:
+            if not isinstance(layer.ff, int):
+                active = layer.ff.top * layer.ff.expert_ff + layer.ff.shared_ff
+                assert abs(active - dense) <= 0.1 * dense
+    assert twice >= 1
